@@ -1152,7 +1152,8 @@ int sd_cache_append(const float* k, int64_t ldk, const float* v, int64_t ldv, vo
  * kv_rank + rot_dim] (row stride ld): the first kv_rank channels normed in place times
  * kv_norm_w, the next rot_dims channels turned as sd_rope_rows does, and the whole row appended
  * to k_cache (one row of kv_rank + rot_dim elements per token: key and value at once).  The
- * same values as sd_rmsnorm_parts + sd_rope_rows + sd_cache_append give.                     */
+ * same values as sd_rmsnorm_parts + sd_rope_rows + sd_cache_append give.  q_latent == NULL:
+ * queries without a latent, only the kv rows are prepared.                                  */
 int sd_latent_prep(float* q_latent, int q_rank, const void* q_norm_w, void* q_bf16,
                    int64_t ld_q_bf16, float* kv, int kv_rank, int rot_dim, const void* kv_norm_w,
                    int64_t ld, int w_f32, float eps, int rot_dims, int rot_layout,
@@ -1225,7 +1226,8 @@ int sd_moe_route_rows(const float* x, int64_t ldx, const void* w_router, int w_f
 size_t sd_moe_experts_scratch_bytes(int n_rows, int top, int E, int F, int W);
 /* out[r*top + j] = down_e(act(gate_e u) * (up_e u)) for e = sel_expert[r, j], u = sel_weight *
  * x[r] (scale_input) or u = x[r] with the result multiplied by the weight (scale_input == 0);
- * act_kind 0: silu.  w_gate_up [E, 2F, W] (gate rows, then up rows), w_down [E, W, F]; x
+ * act_kind 0: silu; act_kind 1: experts of two matrices, down_e(relu(up_e u)^2), w_gate_up then
+ * [E, F, W].  w_gate_up [E, 2F, W] (gate rows, then up rows), w_down [E, W, F]; x
  * [rows, W] (x_bf16, or NULL: the same rows as bf16, same row stride, for the matrix-core path);
  * out [rows*top, W]: the caller adds a row's `top` results.  Rows are grouped by expert on the
  * device; nothing is read back.                                               */
@@ -1239,6 +1241,60 @@ int sd_moe_experts(const float* x, const void* x_bf16, int64_t ldx, const int32_
 int sd_postnorm_residual(float* x, const float* a, int n_a, float sa, const float* b, float sb,
                          const void* w, int w_f32, float eps, void* x_bf16, int n_rows, int W,
                          sd_stream_t stream);
+/* sd_window_softmax_attention with two more masks and a capped score.  chunk > 0: the row at
+ * position i sees only keys j with j / chunk == i / chunk (besides the window and the kept first
+ * tokens' rule; chunks count from position 0 of the sequence).  softcap > 0: a score s (after
+ * `scale`) becomes softcap * tanh(s / softcap).  sinks (f32 [H], or NULL): head h's denominator
+ * also holds exp(sinks[h]), a term without key or value, not scaled and not capped.  A window of
+ * INT32_MAX sees every earlier token.                                                      */
+size_t sd_masked_softmax_attention_scratch_bytes(int n_rows, int H, int dv, int window,
+                                                 int keep_first, int chunk, int max_ctx);
+int sd_masked_softmax_attention(const float* q, int64_t ldq, const void* k_cache,
+                                const void* v_cache, int cache_f32, const int32_t* row_pos,
+                                const int32_t* row_slot, const int32_t* block_tables,
+                                int max_blocks, int page, int n_rows, int H, int G, int dk, int dv,
+                                int window, int keep_first, int chunk, float scale, float softcap,
+                                const float* sinks, float* out, void* out_bf16, void* scratch,
+                                size_t scratch_bytes, sd_stream_t stream);
+/* As sd_qk_norm_append, but every head of q [rows, H*dk] and of k [rows, G*dk] is normed by
+ * itself over its dk channels, with one weight [dk] for all query heads and one for all key
+ * heads.                                                                                   */
+int sd_qk_head_norm_append(float* q, int H, const void* q_norm_w, float* k, int G, int dk,
+                           const void* k_norm_w, const float* v, int dv, int64_t ld, int w_f32,
+                           float eps, void* k_cache, void* v_cache, const int32_t* row_pos,
+                           const int32_t* row_slot, const int32_t* block_tables, int max_blocks,
+                           int page, int n_rows, sd_stream_t stream);
+/* y[r, h, :] *= sigmoid(z[r, h]) in place: one gate per (row, head); y [rows, H*dv] (row stride
+ * ldy), z [rows, H] (row stride ldz); y_bf16 (or NULL, row stride ldyb): the result as bf16. */
+int sd_head_gate_rows(float* y, int64_t ldy, const float* z, int64_t ldz, void* y_bf16,
+                      int64_t ldyb, int n_rows, int H, int dv, int round_bf16_out,
+                      sd_stream_t stream);
+/* A feed-forward's activation: act_kind 0 relu(gate) * up, 1 silu(gate) * up, 2 relu(gate)^2 (up
+ * unused); gate, up [rows, F] (row stride ld).  out (f32, row stride ldo; may be gate itself) and
+ * out_bf16 (row stride ldob) receive it; either may be NULL.                               */
+int sd_act_rows(const float* gate, const float* up, int64_t ld, float* out, int64_t ldo,
+                void* out_bf16, int64_t ldob, int n_rows, int F, int act_kind, int round_bf16_out,
+                sd_stream_t stream);
+/* sd_moe_route_rows with weights = chosen / (sum + renorm_eps) (when renorm) * weight_scale, and
+ * n_gate further products of the same input, computed as the router's are:
+ * gate_out[r, j] = x[r] . w_gate[j] (w_gate [n_gate, K], gate_out f32 [rows, n_gate]).        */
+int sd_moe_route_rows_gated(const float* x, int64_t ldx, const void* w_router, int w_f32,
+                            float* logits, int32_t* sel_expert, float* sel_weight, int n_rows,
+                            int E, int K, int top, int score_kind, int renorm, float renorm_eps,
+                            float weight_scale, const void* w_gate, int n_gate, float* gate_out,
+                            sd_stream_t stream);
+/* The residual update of a layer normed before and after its sublayers, and the norm that
+ * follows, in one launch per row:
+ *   t = a[r*n_a] + ... + a[r*n_a + n_a - 1] (+ sigmoid(b_gate[r*ldg]) * b[r]; b_gate NULL: + b[r]);
+ *   x[r] += rms_norm(t) * w_post                      (a == NULL: x stays)
+ *   x_copy[r] = x[r]                                  (x_copy != NULL)
+ *   x[r] += add                                       (add [W] != NULL)
+ *   h[r] = rms_norm(x[r]) * w_next, h_bf16 the same   (w_next != NULL)
+ * All weights plain, in the model's element type.                                          */
+int sd_residual_norm(float* x, const float* a, int n_a, const float* b, const float* b_gate,
+                     int64_t ldg, const void* w_post, const void* add, const void* w_next,
+                     int w_f32, float eps, float* x_copy, float* h, void* h_bf16, int n_rows,
+                     int W, sd_stream_t stream);
 /* x[r, c] *= s                                                                             */
 int sd_scale_rows(float* x, int64_t ld, float s, int n_rows, int n_cols, sd_stream_t stream);
 
@@ -1247,12 +1303,14 @@ typedef enum {
   SD_MIX_CHANNEL_DECAY = 1, /* recurrence with an input-dependent decay per key channel */
   SD_MIX_WINDOW_POOL = 2,   /* sd_window_pool_attention */
   SD_MIX_LATENT = 3,        /* softmax window attention over latent keys / values */
-  SD_MIX_SOFTMAX_SSD = 4    /* softmax window attention and a state-space recurrence side by side */
+  SD_MIX_SOFTMAX_SSD = 4,   /* softmax window attention and a state-space recurrence side by side */
+  SD_MIX_SOFTMAX = 5        /* grouped-query softmax attention (sd_masked_softmax_attention), no rotation */
 } sd_mixer_kind;
 
 typedef enum {
   SD_BLOCK_GATED = 0,       /* h = norm(x); x += sigmoid(r1) mixer(h) + sigmoid(r2) ff(h) */
-  SD_BLOCK_POSTNORM = 1     /* x += norm1(mixer(x)); x += norm2(ff(x)) */
+  SD_BLOCK_POSTNORM = 1,    /* x += norm1(mixer(x)); x += norm2(ff(x)) */
+  SD_BLOCK_SANDWICH = 2     /* x += post_norm(mixer(norm(x))); x += post_norm2(ff(norm2(x))) */
 } sd_block_kind;
 
 /* One layer: h = norm(x); x += sigmoid(r1) * mixer(h) + sigmoid(r2) * ff(h).  w_in stacks every
@@ -1327,6 +1385,35 @@ typedef struct {
   const void* w_router;     /* [n_experts, width] */
   const void* w_gate_up;    /* [n_experts, 2*expert_ff, width] */
   const void* w_down_e;     /* [n_experts, width, expert_ff] */
+  /* ---- SD_BLOCK_SANDWICH layers (all zero otherwise): a plain norm before and after each
+   * sublayer.  norm_w / norm2_w come before the mixer / the feed-forward, post_norm_w /
+   * post_norm2_w after them.  w_in stacks the matrices that read norm(x): SD_MIX_LATENT with
+   * q_rank == 0 (queries straight from the input): q [heads*(dim+rot_dim)], dkv [kv_rank +
+   * rot_dim], then the head gates [heads] when head_gate; SD_MIX_SOFTMAX: q [heads*dim],
+   * k [kv_heads*dim], v [kv_heads*vdim].  The feed-forward is absent (ff == 0, n_experts == 0),
+   * dense (ff > 0: w_ff_in [2*ff, width] gate rows then up rows, w_down [width, ff], ff_act as
+   * sd_act_rows) or routed experts (the fields above, plus the ones below).                  */
+  const void* post_norm_w;  /* [width] */
+  const void* post_norm2_w; /* [width] or NULL (no feed-forward) */
+  const void* pre_add;      /* [width] (model element type) or NULL: added to the stream before the layer */
+  int chunk;                /* keys of the row's own chunk of this many positions only; 0: no chunks */
+  float softcap;            /* 0: scores are not capped */
+  const float* sinks;       /* f32 [heads] or NULL */
+  int head_gate;            /* a head's output is multiplied by the sigmoid of its gate row's product */
+  int qk_head_norm;         /* q_norm_w / k_norm_w are [dim], applied per head */
+  const void* w_ff_in;
+  const void* w_ff_in_tiled;
+  int ff_act;
+  int expert_act;           /* sd_moe_experts act_kind */
+  int route_score, route_renorm, expert_scale_input;
+  float route_renorm_eps, route_scale;
+  int shared_ff;            /* an expert every token uses: down(act(in h)) * sigmoid(gate . h); 0: none */
+  int shared_act;           /* as sd_act_rows */
+  const void* w_shared_in;  /* [shared_ff, width] (gated activations: [2*shared_ff, width]) */
+  const void* w_shared_in_tiled;
+  const void* w_shared_down; /* [width, shared_ff] */
+  const void* w_shared_down_tiled;
+  const void* w_shared_gate; /* [1, width] or NULL: no gate */
 } sd_seq_layer;
 
 typedef struct {

@@ -93,7 +93,13 @@ class SeqLayer(C.Structure):
                 ("s_norm_groups", i32), ("conv_w", vp), ("conv_b", vp), ("dt_bias", vp), ("a_log", vp),
                 ("skip_d", vp), ("s_norm_w", vp), ("w_o2", vp), ("w_o2_tiled", vp), ("conv_state", vp),
                 ("n_experts", i32), ("top", i32), ("expert_ff", i32), ("w_router", vp), ("w_gate_up", vp),
-                ("w_down_e", vp)]
+                ("w_down_e", vp),
+                ("post_norm_w", vp), ("post_norm2_w", vp), ("pre_add", vp), ("chunk", i32), ("softcap", C.c_float),
+                ("sinks", vp), ("head_gate", i32), ("qk_head_norm", i32), ("w_ff_in", vp), ("w_ff_in_tiled", vp),
+                ("ff_act", i32), ("expert_act", i32), ("route_score", i32), ("route_renorm", i32),
+                ("expert_scale_input", i32), ("route_renorm_eps", C.c_float), ("route_scale", C.c_float),
+                ("shared_ff", i32), ("shared_act", i32), ("w_shared_in", vp), ("w_shared_in_tiled", vp),
+                ("w_shared_down", vp), ("w_shared_down_tiled", vp), ("w_shared_gate", vp)]
 
 
 class SeqModelDesc(C.Structure):
@@ -258,6 +264,16 @@ SIGNATURES = {
     "sd_moe_experts": (i32, [vp, vp, i64, vp, vp, vp, vp, i32, vp, i32, i32, i32, i32, i32, i32, i32, vp, C.c_size_t, vp]),
     "sd_postnorm_residual": (i32, [vp, vp, i32, C.c_float, vp, C.c_float, vp, i32, C.c_float, vp, i32, i32, vp]),
     "sd_scale_rows": (i32, [vp, i64, C.c_float, i32, i32, vp]),
+    "sd_masked_softmax_attention_scratch_bytes": (C.c_size_t, [i32, i32, i32, i32, i32, i32, i32]),
+    "sd_masked_softmax_attention": (i32, [vp, i64, vp, vp, i32, vp, vp, vp, i32, i32, i32, i32, i32, i32, i32, i32,
+                                          i32, i32, C.c_float, C.c_float, vp, vp, vp, vp, C.c_size_t, vp]),
+    "sd_qk_head_norm_append": (i32, [vp, i32, vp, vp, i32, i32, vp, vp, i32, i64, i32, C.c_float, vp, vp, vp, vp, vp,
+                                     i32, i32, i32, vp]),
+    "sd_head_gate_rows": (i32, [vp, i64, vp, i64, vp, i64, i32, i32, i32, i32, vp]),
+    "sd_act_rows": (i32, [vp, vp, i64, vp, i64, vp, i64, i32, i32, i32, i32, vp]),
+    "sd_moe_route_rows_gated": (i32, [vp, i64, vp, i32, vp, vp, vp, i32, i32, i32, i32, i32, i32, C.c_float, C.c_float,
+                                      vp, i32, vp, vp]),
+    "sd_residual_norm": (i32, [vp, vp, i32, vp, vp, i64, vp, vp, vp, i32, C.c_float, vp, vp, vp, i32, i32, vp]),
     "sd_seq_model_create": (vp, [C.POINTER(SeqModelDesc)]),
     "sd_seq_model_destroy": (None, [vp]),
     "sd_seq_model_workspace_bytes": (C.c_size_t, [vp, i32, i32, i32]),

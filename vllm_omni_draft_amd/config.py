@@ -210,7 +210,7 @@ def rope_table(cfg: ModelConfig, device="cpu") -> torch.Tensor:
 
 # ---------------------------------------------------------------------------------------------
 # Decoders described layer by layer (recurrent and windowed mixers); served by seq_engine.SeqEngine.
-MIXER_KINDS = ("retention", "gla", "attention", "latent_attention", "parallel")
+MIXER_KINDS = ("retention", "gla", "attention", "latent_attention", "parallel", "softmax_attention")
 
 
 @dataclass
@@ -247,19 +247,29 @@ class ExpertsSpec:
     """Routed experts as a layer's feed-forward: `top` of `experts` gated feed-forwards of width
     `ff` per token.  score: "sigmoid" or "softmax" over the router's logits; renorm: the chosen
     weights are divided by their sum; scale_input: the weight multiplies the expert's input
-    (else its output)."""
+    (else its output).  act "silu": an expert is down(silu(gate h) * (up h)); "relu2": an expert has
+    two matrices, down(relu(up h)^2).  The chosen weights are divided by (their sum + renorm_eps)
+    when renorm, then multiplied by scale.  shared_ff > 0: one more expert of that width and the
+    same form runs for every token and is added, times sigmoid(g . h) when shared_gate."""
     experts: int
     top: int
     ff: int
     score: str = "sigmoid"
     renorm: bool = False
     scale_input: bool = True
+    act: str = "silu"
+    renorm_eps: float = 0.0
+    scale: float = 1.0
+    shared_ff: int = 0
+    shared_gate: bool = True
 
     def validate(self) -> None:
-        if self.experts < 1 or not 1 <= self.top <= self.experts or self.ff < 1:
-            raise ValueError(f"experts {self.experts}, top {self.top}, ff {self.ff}")
+        if self.experts < 1 or not 1 <= self.top <= self.experts or self.ff < 1 or self.shared_ff < 0:
+            raise ValueError(f"experts {self.experts}, top {self.top}, ff {self.ff}, shared ff {self.shared_ff}")
         if self.score not in ("sigmoid", "softmax"):
             raise ValueError(f"unknown router score {self.score!r}")
+        if self.act not in ("silu", "relu2"):
+            raise ValueError(f"unknown expert activation {self.act!r}")
 
 
 @dataclass
@@ -274,7 +284,13 @@ class MixerSpec:
     shared by the heads (queries through a latent of q_rank channels; dim counts the unrotated
     channels of a head); "parallel": grouped-query softmax attention without rotation, q and k
     normed over the whole projection, over a window that also keeps the first keep_first tokens,
-    beside a state-space recurrence (ssd) on the same input, summed with two scales."""
+    beside a state-space recurrence (ssd) on the same input, summed with two scales;
+    "softmax_attention": grouped-query softmax attention without rotation, q and k normed per
+    head with one weight of `dim` channels each (qk_head_norm), scores capped by softcap *
+    tanh(s / softcap), keys of the query's own chunk of `chunk` positions only.  A latent
+    attention with q_rank 0 projects its queries straight from the input; window 0 sees every
+    earlier token; sink: a learned term per head in the softmax's denominator; head_gate: a
+    head's output is multiplied by the sigmoid of a product of the input."""
     kind: str
     heads: int
     dim: int
@@ -297,6 +313,11 @@ class MixerSpec:
     ssd: Optional[SsdSpec] = None  # parallel
     left_scale: float = 1.0        # parallel: factor of the attention
     right_scale: float = 1.0       # parallel: factor of the recurrence
+    chunk: int = 0                 # softmax attention: keys of the query's own chunk only (0: no chunks)
+    softcap: float = 0.0           # scores capped by softcap * tanh(s / softcap) (0: not capped)
+    sink: bool = False             # a learned term per head in the softmax's denominator
+    head_gate: bool = False        # outputs gated per head
+    qk_head_norm: bool = False     # q and k normed per head
 
     def validate(self) -> None:
         if self.kind not in MIXER_KINDS:
@@ -308,12 +329,16 @@ class MixerSpec:
         if self.rot_layout not in ("half", "interleaved"):
             raise ValueError(f"unknown rotary layout {self.rot_layout!r}")
         if self.kind == "latent_attention":
-            if min(self.q_rank, self.kv_rank) < 1 or self.rot_dim < 0 or self.window < 1:
-                raise ValueError("latent attention needs q_rank, kv_rank >= 1, rot_dim >= 0, window >= 1")
+            if self.q_rank < 0 or self.kv_rank < 1 or self.rot_dim < 0 or self.window < 0:
+                raise ValueError("latent attention needs q_rank >= 0, kv_rank >= 1, rot_dim >= 0, window >= 0")
             if self.rot_dims < 0 or self.rot_dims % 2 or self.rot_dims > self.rot_dim:
                 raise ValueError(f"rot_dims {self.rot_dims} must be even and at most rot_dim {self.rot_dim}")
             if self.kv_rank > 512 or self.kv_heads != self.heads:
                 raise ValueError("latent attention: kv_rank above 512, or kv_heads given")
+            return
+        if self.kind == "softmax_attention":
+            if self.window < 0 or self.chunk < 0 or self.softcap < 0 or self.rot_dims or self.vdim > 512:
+                raise ValueError("softmax attention needs window >= 0, chunk >= 0, softcap >= 0, no rotation, vdim <= 512")
             return
         if self.kind == "parallel":
             if self.window < 1 or self.keep_first < 0 or self.rot_dims or self.ssd is None or self.vdim > 512:
@@ -367,6 +392,7 @@ class SeqLayerSpec:
     mixer: MixerSpec
     ff: int = 0                    # width of the gated feed-forward beside the mixer; 0: none
     experts: Optional[ExpertsSpec] = None   # routed experts as the feed-forward
+    ff_act: str = "relu"           # the gated feed-forward's activation: "relu" or "silu"
 
 
 @dataclass
@@ -382,17 +408,61 @@ class SeqModelConfig:
     name: str = "custom"
     # "gated": the layer above.  "postnorm": x += norm1(mixer(x)); x += norm2(ff(x)), plain norm
     # weights, the sublayers read x itself; the feed-forward is a set of routed experts or absent.
+    # "sandwich": x += norm1b(mixer(norm1(x))); x += norm2b(ff(norm2(x))), plain norm weights; the
+    # feed-forward is gated, a set of routed experts (with or without a shared one), or absent.
     block: str = "gated"
     embed_scale: float = 1.0
     bigram: Optional[dict] = None  # {buckets, mul_prev, mul_cur}: a hashed table of token pairs added to the embedding
     tied_head: bool = True         # False: the output head is its own tensor
     logit_scale: float = 1.0
+    # {start, stop, times}: layers start .. stop-1 run `times` times in a row with the same weights
+    # (every pass keeps a cache of its own); the learned vector 'loop.step'[t] is added to the
+    # stream before pass t.
+    loop: Optional[dict] = None
+
+    @property
+    def runs(self) -> List[tuple]:
+        """The layers in the order they run: (layer, pass) pairs, pass None outside the repeated span."""
+        n = len(self.layers)
+        if not self.loop:
+            return [(i, None) for i in range(n)]
+        a, b, t = int(self.loop["start"]), int(self.loop["stop"]), int(self.loop["times"])
+        return ([(i, None) for i in range(a)] + [(i, p) for p in range(t) for i in range(a, b)]
+                + [(i, None) for i in range(b, n)])
+
+    @property
+    def n_runs(self) -> int:
+        return len(self.runs)
+
+    def _validate_sandwich(self) -> None:
+        for l in self.layers:
+            l.mixer.validate()
+            if l.mixer.kind not in ("latent_attention", "softmax_attention"):
+                raise ValueError(f"mixer {l.mixer.kind!r} does not belong to a 'sandwich' model")
+            if l.mixer.kind == "latent_attention" and l.mixer.q_rank:
+                raise ValueError("a 'sandwich' model's latent attention projects its queries straight from the input")
+            if l.mixer.kind == "softmax_attention" and not l.mixer.qk_head_norm:
+                raise ValueError("a 'sandwich' model's softmax attention norms q and k per head")
+            if l.ff < 0 or l.ff_act not in ("relu", "silu") or (l.ff and l.experts is not None):
+                raise ValueError("a layer's feed-forward is gated (ff > 0, relu or silu) or routed experts, not both")
+            if l.experts is not None:
+                l.experts.validate()
+        if self.loop is not None:
+            a, b, t = (int(self.loop[k]) for k in ("start", "stop", "times"))
+            if not 0 <= a < b <= len(self.layers) or t < 1:
+                raise ValueError(f"loop {self.loop}: needs 0 <= start < stop <= layers and times >= 1")
 
     def validate(self) -> None:
         if self.width < 1 or self.vocab < 1 or not self.layers:
             raise ValueError("a model needs width, vocab and at least one layer")
-        if self.block not in ("gated", "postnorm"):
+        if self.block not in ("gated", "postnorm", "sandwich"):
             raise ValueError(f"unknown block {self.block!r}")
+        if self.block == "sandwich":
+            if self.bigram is not None:
+                raise ValueError("a 'sandwich' model has no bigram table")
+            return self._validate_sandwich()
+        if self.loop is not None:
+            raise ValueError("only a 'sandwich' model repeats a span of its layers")
         if self.bigram is not None and int(self.bigram["buckets"]) < 1:
             raise ValueError("a bigram table needs buckets >= 1")
         for l in self.layers:
@@ -419,8 +489,24 @@ class SeqModelConfig:
             n += self.vocab * W
         if self.bigram:
             n += (int(self.bigram["buckets"]) + 1) * W
+        if self.loop:
+            n += int(self.loop["times"]) * W
         for l in self.layers:
             m = l.mixer
+            if self.block == "sandwich":
+                n += 2 * W + (2 * W if (l.ff or l.experts) else 0) + m.heads * m.vdim * W
+                if m.kind == "latent_attention":
+                    n += W * (m.heads * (m.dim + m.rot_dim) + m.kv_rank + m.rot_dim + (m.heads if m.head_gate else 0))
+                    n += m.kv_rank + m.heads * (m.dim + m.vdim) * m.kv_rank + (m.heads if m.sink else 0)
+                else:
+                    n += W * (m.heads * m.dim + m.kv_heads * (m.dim + m.vdim)) + 2 * m.dim
+                n += 3 * l.ff * W
+                ex = l.experts
+                if ex is not None:
+                    per = 3 if ex.act == "silu" else 2
+                    n += ex.experts * (W + per * ex.ff * W) + per * ex.shared_ff * W
+                    n += W if ex.shared_ff and ex.shared_gate else 0
+                continue
             if m.kind == "latent_attention":
                 n += W + W * (m.q_rank + m.kv_rank + m.rot_dim) + m.q_rank + m.kv_rank
                 n += m.heads * ((m.dim + m.rot_dim) * m.q_rank + (m.dim + m.vdim) * m.kv_rank + m.vdim * W)
@@ -531,8 +617,59 @@ def naburax_config(cfg: dict, tensor_shapes: Optional[dict] = None, **overrides)
     return out
 
 
+def fepopel_config(cfg: dict, tensor_shapes: Optional[dict] = None, **overrides) -> SeqModelConfig:
+    """A Fepopel config.json: layers normed before and after each sublayer; latent attention over
+    every earlier token (queries straight from the input, a learned sink per head in the softmax,
+    outputs gated per head) and grouped-query softmax attention inside chunks (q and k normed per
+    head, capped scores, no rotation), in any order; a gated feed-forward, routed experts of two
+    matrices beside a gated shared expert, or none; a span of layers that runs several times over;
+    a scaled embedding and an untied head."""
+    layers = []
+    for i, l in enumerate(cfg["layers"]):
+        m, kind = l["mixer"], l["type"]
+        if kind == "latent_attention":
+            rot = m.get("rot") or {}
+            rot_dim = int(m.get("rot_dim", 0))
+            spec = MixerSpec(kind=kind, heads=int(m["heads"]), dim=int(m["dim"]), vdim=int(m["vdim"]), q_rank=0,
+                             kv_rank=int(m["kv_rank"]), rot_dim=rot_dim, rot_dims=int(rot.get("dims", rot_dim)),
+                             rot_base=float(rot.get("base", 10000.0)), rot_layout="interleaved",
+                             scale=float(m["scale"]), window=0, sink=True, head_gate=True)
+        elif kind == "attention":
+            mask = m.get("mask") or {}
+            spec = MixerSpec(kind="softmax_attention", heads=int(m["heads"]), kv_heads=int(m.get("kv_heads", 0)),
+                             dim=int(m["dim"]), vdim=int(m["vdim"]), scale=float(m["scale"]), window=0,
+                             chunk=int(mask.get("size", 0)), softcap=float(m.get("softcap", 0.0)), qk_head_norm=True)
+        else:
+            raise ValueError(f"layer {i}: unknown mixer type {kind!r}")
+        mlp = l.get("mlp")
+        ff, experts = 0, None
+        if mlp:
+            mk = mlp.get("kind", "dense")
+            if mk == "dense":
+                ff = int(mlp["ff"])
+            elif mk == "moe":
+                r, sh = mlp["router"], mlp.get("shared")
+                experts = ExpertsSpec(experts=int(r["experts"]), top=int(r["top"]), ff=int(mlp["expert"]["ff"]),
+                                      score="softmax", renorm=True, scale_input=False, act="relu2", renorm_eps=1e-20,
+                                      scale=float(r.get("scale", 1.0)), shared_ff=int(sh["ff"]) if sh else 0)
+            else:
+                raise ValueError(f"layer {i}: feed-forward kind {mk!r} is not supported")
+        layers.append(SeqLayerSpec(spec, ff, experts, ff_act="silu"))
+    emb, loop = cfg.get("embedding") or {}, cfg.get("loop")
+    out = SeqModelConfig(arch="fepopel", width=int(cfg["width"]), vocab=int(cfg["vocab"]), layers=layers,
+                         norm_eps=float(cfg["norm"]["eps"]), name=cfg.get("architecture", "Fepopel"),
+                         block="sandwich", embed_scale=float(emb.get("scale", 1.0)), tied_head=False,
+                         loop={k: int(loop[k]) for k in ("start", "stop", "times")} if loop else None)
+    for k, v in overrides.items():
+        if not hasattr(out, k):
+            raise ValueError(f"Unknown config parameter: {k}")
+        setattr(out, k, v)
+    out.validate()
+    return out
+
+
 # config.json "architecture" -> builder of a layer-list config
-SEQ_ARCHITECTURES = {"Puguzen": puguzen_config, "Naburax": naburax_config}
+SEQ_ARCHITECTURES = {"Puguzen": puguzen_config, "Naburax": naburax_config, "Fepopel": fepopel_config}
 
 
 def safetensors_shapes(path: str) -> dict:

@@ -997,6 +997,7 @@ inline size_t al(size_t v) { return (v + 255) & ~(size_t)255; }
 constexpr int kWideRows = 256;  // rows one call of the many-row linear family takes
 struct SeqWs {
   size_t x, h, proj, dec, o, y, mix, ffo, hout, hb, yb, actb, houtb, wide, wide_bytes, attn, attn_bytes, total;
+  size_t sg;   // a shared expert's gate per row
   // layers normed on their output
   size_t pq, qe, cqb, conv, step, decay, rlog, sel_e, sel_w, dn, moe, moe_bytes;
 };
@@ -1004,6 +1005,27 @@ struct SeqWs {
 struct PnCols {
   int dq, dkv, q, k, v, z, xbc, dt, total, inner, conv_ch;
 };
+// column offsets inside the fused input projection of a layer normed before and after its sublayers
+struct SwCols {
+  int q, dkv, g, k, v, total;
+};
+SwCols sw_cols(const sd_seq_layer& l) {
+  SwCols c = {};
+  int at = 0;
+  if (l.kind == SD_MIX_LATENT) {
+    c.q = at;   at += l.heads * (l.dim + l.rot_dim);
+    c.dkv = at; at += l.kv_rank + l.rot_dim;
+    c.g = at;   at += l.head_gate ? l.heads : 0;
+  } else {
+    c.q = at; at += l.heads * l.dim;
+    c.k = at; at += l.kv_heads * l.dim;
+    c.v = at; at += l.kv_heads * l.vdim;
+  }
+  c.total = at;
+  return c;
+}
+inline int act_inputs(int act_kind) { return act_kind == 2 ? 1 : 2; }   // matrices an activation of sd_act_rows reads
+constexpr int kNoWindow = 0x7fffffff;
 PnCols pn_cols(const sd_seq_layer& l) {
   PnCols c = {};
   int at = 0;
@@ -1035,6 +1057,37 @@ SeqWs plan_seq(const sd_seq_model& m, int rows, int n_out, int max_ctx) {
     wide = n > wide ? n : wide;
   };
   for (const sd_seq_layer& l : m.layers) {
+    if (l.block == SD_BLOCK_SANDWICH) {
+      const SwCols c = sw_cols(l);
+      up(proj, (size_t)c.total);
+      need(l.w_in_tiled, wr, c.total, W);
+      need(l.w_o_tiled, wr, W, l.heads * l.vdim);
+      up(hv, (size_t)l.heads * l.vdim);
+      up(attn, sd_masked_softmax_attention_scratch_bytes(rows, l.heads, l.kind == SD_MIX_LATENT ? l.kv_rank : l.vdim,
+                                                         l.window, 0, l.chunk, max_ctx));
+      if (l.kind == SD_MIX_LATENT) {
+        up(qe, (size_t)l.heads * (l.kv_rank + l.rot_dim));
+        up(hv, (size_t)l.heads * l.kv_rank);
+      }
+      if (l.ff > 0) {
+        up(proj, (size_t)act_inputs(l.ff_act) * l.ff);
+        up(ff, (size_t)l.ff);
+        need(l.w_ff_in_tiled, wr, act_inputs(l.ff_act) * l.ff, W);
+        need(l.w_down_tiled, wr, W, l.ff);
+      }
+      if (l.n_experts > 0) {
+        up(ne, (size_t)l.n_experts);
+        up(top, (size_t)l.top);
+        up(moe, sd_moe_experts_scratch_bytes(rows, l.top, l.n_experts, l.expert_ff, W));
+      }
+      if (l.shared_ff > 0) {
+        up(proj, (size_t)act_inputs(l.shared_act) * l.shared_ff);
+        up(ff, (size_t)l.shared_ff);
+        need(l.w_shared_in_tiled, wr, act_inputs(l.shared_act) * l.shared_ff, W);
+        need(l.w_shared_down_tiled, wr, W, l.shared_ff);
+      }
+      continue;
+    }
     if (l.block == SD_BLOCK_POSTNORM) {
       const PnCols c = pn_cols(l);
       up(proj, (size_t)c.total);
@@ -1111,6 +1164,7 @@ SeqWs plan_seq(const sd_seq_model& m, int rows, int n_out, int max_ctx) {
   w.dn = off;    off += al(R * top * W * f);
   w.moe_bytes = moe;
   w.moe = off;   off += al(moe ? moe : 16);
+  w.sg = off;    off += al(R * f);
   w.total = off;
   return w;
 }
@@ -1146,8 +1200,23 @@ extern "C" sd_seq_model* sd_seq_model_create(const sd_seq_model_desc* desc) {
   for (int i = 0; i < desc->n_layers; ++i) {
     const sd_seq_layer& l = m->layers[i];
     const char* bad = nullptr;
+    if (l.block == SD_BLOCK_SANDWICH) {
+      if (l.kind != SD_MIX_LATENT && l.kind != SD_MIX_SOFTMAX) bad = "a layer normed before and after its sublayers takes latent or grouped-query softmax attention";
+      else if (i > 0 && m->layers[i - 1].block != SD_BLOCK_SANDWICH) bad = "it follows a layer of another kind";
+      else if (l.heads < 1 || l.dim < 1 || l.vdim < 1 || l.window < 1 || l.chunk < 0 || l.softcap < 0.f) bad = "head counts / sizes / window / chunk / cap";
+      else if (!l.norm_w || !l.post_norm_w || !(l.w_in || l.w_in_tiled) || !(l.w_o || l.w_o_tiled) || !l.k_cache) bad = "a null weight or cache";
+      else if ((l.w_in_tiled || l.w_o_tiled || l.w_ff_in_tiled || l.w_down_tiled || l.w_shared_in_tiled || l.w_shared_down_tiled) && desc->weights_f32) bad = "tiled matrices are bf16";
+      else if (l.kind == SD_MIX_LATENT && (l.q_rank != 0 || l.kv_rank < 1 || l.kv_rank > 512 || l.rot_dim < 0 || l.rot_dims < 0 || l.rot_dims > l.rot_dim ||
+               l.rot_dims % 2 || (l.rot_dims && !l.inv_freq) || !l.dkv_norm_w || !l.w_uk_t || !l.w_uv)) bad = "latent size / rotary dims / a null latent weight";
+      else if (l.kind == SD_MIX_SOFTMAX && (l.kv_heads < 1 || l.heads % l.kv_heads || l.vdim > 512 || !l.v_cache || !l.qk_head_norm || !l.q_norm_w || !l.k_norm_w)) bad = "attention needs kv heads that divide the heads, vdim <= 512, a value cache and per-head norms";
+      else if (l.ff < 0 || (l.ff > 0 && (l.n_experts > 0 || l.ff_act < 0 || l.ff_act > 2 || !(l.w_ff_in || l.w_ff_in_tiled) || !(l.w_down || l.w_down_tiled)))) bad = "a dense feed-forward needs its two matrices and a known activation, and excludes experts";
+      else if (l.n_experts > 0 && (l.top < 1 || l.top > l.n_experts || l.expert_ff < 1 || !l.w_router || !l.w_gate_up || !l.w_down_e || l.expert_act < 0 || l.expert_act > 1)) bad = "routed experts need top <= experts, their matrices and a known activation";
+      else if (l.shared_ff < 0 || (l.shared_ff > 0 && (l.n_experts < 1 || l.shared_act < 0 || l.shared_act > 2 || !(l.w_shared_in || l.w_shared_in_tiled) || !(l.w_shared_down || l.w_shared_down_tiled)))) bad = "a shared expert stands beside routed experts and needs its matrices";
+      else if ((l.ff > 0 || l.n_experts > 0) && (!l.norm2_w || !l.post_norm2_w)) bad = "a feed-forward needs its two norms";
+    } else
     if (l.block == SD_BLOCK_POSTNORM) {
       if (l.kind != SD_MIX_LATENT && l.kind != SD_MIX_SOFTMAX_SSD) bad = "a layer normed on its output takes latent attention or attention beside a state-space recurrence";
+      else if (i > 0 && m->layers[i - 1].block == SD_BLOCK_SANDWICH) bad = "it follows a layer normed before and after its sublayers";
       else if (l.heads < 1 || l.dim < 1 || l.vdim < 1 || l.window < 1 || l.keep_first < 0) bad = "head counts / sizes / window";
       else if (!l.norm_w || !(l.w_in || l.w_in_tiled) || !(l.w_o || l.w_o_tiled) || !l.k_cache) bad = "a null weight or cache";
       else if ((l.w_in_tiled || l.w_o_tiled || l.w_uq_tiled || l.w_o2_tiled) && desc->weights_f32) bad = "tiled matrices are bf16";
@@ -1297,6 +1366,111 @@ int postnorm_layer(const sd_seq_model& m, const sd_seq_layer& l, const sd_seq_ba
   }
   return SD_OK;
 }
+
+// One layer normed before and after its sublayers: x += post_norm(mixer(norm(x))); x +=
+// post_norm2(ff(norm2(x))).  On entry h / hb hold norm(x + pre_add) already (the layer before, or
+// the caller, left them); on return they hold the next layer's, or nothing after the last.
+int sandwich_layer(const sd_seq_model& m, const sd_seq_layer& l, const sd_seq_layer* next, const sd_seq_batch& b,
+                   char* base, const SeqWs& w, float* x_copy, sd_stream_t stream) {
+  const sd_seq_model_desc& d = m.d;
+  const int W = d.width, R = b.n_rows, f32 = d.weights_f32, rnd = !f32;
+  const float eps = d.norm_eps;
+  float* x = (float*)(base + w.x);
+  float* h = (float*)(base + w.h);
+  float* proj = (float*)(base + w.proj);
+  float* o = (float*)(base + w.o);
+  float* y = (float*)(base + w.y);
+  float* mix = (float*)(base + w.mix);
+  float* ffo = (float*)(base + w.ffo);
+  bf16_t* hb = (bf16_t*)(base + w.hb);
+  bf16_t* yb = (bf16_t*)(base + w.yb);
+  bf16_t* actb = (bf16_t*)(base + w.actb);
+  void* wide_ws = base + w.wide;
+  const SwCols c = sw_cols(l);
+  const int64_t ld = c.total;
+  const int H = l.heads, dk = l.dim, dv = l.vdim;
+  const void* next_add = next ? next->pre_add : nullptr;
+  const void* next_norm = next ? next->norm_w : nullptr;
+  const bool has_ff = l.ff > 0 || l.n_experts > 0;
+  SQ_TRY(seq_linear(l.w_in, l.w_in_tiled, f32, h, nullptr, W, hb, W, nullptr, proj, ld, R, c.total, W, wide_ws,
+                    w.wide_bytes, stream));
+  if (l.kind == SD_MIX_LATENT) {
+    const int rk = l.kv_rank, dr = l.rot_dim, dh = dk + dr, de = rk + dr;
+    float* qe = (float*)(base + w.qe);
+    // the latent normed, the shared rotated key part turned, the row [latent | rotated part] cached
+    SQ_TRY(sd_latent_prep(nullptr, 0, nullptr, nullptr, 0, proj + c.dkv, rk, dr, l.dkv_norm_w, ld, f32, eps, l.rot_dims,
+                          l.rot_layout, l.inv_freq, l.rot_mag, l.k_cache, b.row_pos, b.row_slot, b.block_tables,
+                          b.max_blocks, b.page, R, stream));
+    // a head's query against the latent: its key expansion, transposed, applied to the unrotated
+    // part; the rotated part is turned into place behind it
+    SQ_TRY(sd_matmul_rows_batched(proj + c.q, ld, dh, l.w_uk_t, f32, (int64_t)rk * dk, qe, (int64_t)H * de, de, nullptr,
+                                  R, rk, dk, H, stream));
+    if (dr > 0)
+      SQ_TRY(sd_rope_copy_rows(proj + c.q, ld, dh, dk, qe, (int64_t)H * de, de, rk, b.row_pos, R, H, dr, l.rot_dims,
+                               l.rot_layout, l.inv_freq, l.rot_mag, stream));
+    SQ_TRY(sd_masked_softmax_attention(qe, (int64_t)H * de, l.k_cache, nullptr, f32, b.row_pos, b.row_slot,
+                                       b.block_tables, b.max_blocks, b.page, R, H, 1, de, rk, l.window, 0, l.chunk,
+                                       l.score_scale, l.softcap, l.sinks, o, nullptr, base + w.attn, w.attn_bytes,
+                                       stream));
+    // a head's value expansion applied to its weighted latent, then the head's gate
+    bf16_t* y_b = l.w_o_tiled ? yb : nullptr;
+    SQ_TRY(sd_matmul_rows_batched(o, (int64_t)H * rk, rk, l.w_uv, f32, (int64_t)dv * rk, y, (int64_t)H * dv, dv,
+                                  l.head_gate ? nullptr : y_b, R, dv, rk, H, stream));
+    if (l.head_gate)
+      SQ_TRY(sd_head_gate_rows(y, (int64_t)H * dv, proj + c.g, ld, y_b, (int64_t)H * dv, R, H, dv, rnd, stream));
+    SQ_TRY(seq_linear(l.w_o, l.w_o_tiled, f32, y, nullptr, (int64_t)H * dv, yb, (int64_t)H * dv, nullptr, mix, W, R, W,
+                      H * dv, wide_ws, w.wide_bytes, stream));
+  } else {
+    const int G = l.kv_heads;
+    SQ_TRY(sd_qk_head_norm_append(proj + c.q, H, l.q_norm_w, proj + c.k, G, dk, l.k_norm_w, proj + c.v, dv, ld, f32, eps,
+                                  l.k_cache, l.v_cache, b.row_pos, b.row_slot, b.block_tables, b.max_blocks, b.page,
+                                  R, stream));
+    SQ_TRY(sd_masked_softmax_attention(proj + c.q, ld, l.k_cache, l.v_cache, f32, b.row_pos, b.row_slot,
+                                       b.block_tables, b.max_blocks, b.page, R, H, G, dk, dv, l.window, 0, l.chunk,
+                                       l.score_scale, l.softcap, l.sinks, o, l.w_o_tiled ? yb : nullptr,
+                                       base + w.attn, w.attn_bytes, stream));
+    SQ_TRY(seq_linear(l.w_o, l.w_o_tiled, f32, o, nullptr, (int64_t)H * dv, yb, (int64_t)H * dv, nullptr, mix, W, R, W,
+                      H * dv, wide_ws, w.wide_bytes, stream));
+  }
+  if (!has_ff)
+    return sd_residual_norm(x, mix, 1, nullptr, nullptr, 0, l.post_norm_w, next_add, next_norm, f32, eps, x_copy, h, hb,
+                            R, W, stream);
+  SQ_TRY(sd_residual_norm(x, mix, 1, nullptr, nullptr, 0, l.post_norm_w, nullptr, l.norm2_w, f32, eps, nullptr, h, hb, R,
+                          W, stream));
+  if (l.ff > 0) {
+    const int F = l.ff, n_in = act_inputs(l.ff_act);
+    SQ_TRY(seq_linear(l.w_ff_in, l.w_ff_in_tiled, f32, h, nullptr, W, hb, W, nullptr, proj, (int64_t)n_in * F, R,
+                      n_in * F, W, wide_ws, w.wide_bytes, stream));
+    SQ_TRY(sd_act_rows(proj, n_in > 1 ? proj + F : nullptr, (int64_t)n_in * F, proj, (int64_t)n_in * F,
+                       l.w_down_tiled ? actb : nullptr, F, R, F, l.ff_act, rnd, stream));
+    SQ_TRY(seq_linear(l.w_down, l.w_down_tiled, f32, proj, nullptr, (int64_t)n_in * F, actb, F, nullptr, ffo, W, R, W,
+                      F, wide_ws, w.wide_bytes, stream));
+    return sd_residual_norm(x, ffo, 1, nullptr, nullptr, 0, l.post_norm2_w, next_add, next_norm, f32, eps, x_copy, h,
+                            hb, R, W, stream);
+  }
+  float* rlog = (float*)(base + w.rlog);
+  int32_t* sel_e = (int32_t*)(base + w.sel_e);
+  float* sel_w = (float*)(base + w.sel_w);
+  float* dn = (float*)(base + w.dn);
+  float* sg = (float*)(base + w.sg);
+  const bool gated_shared = l.shared_ff > 0 && l.w_shared_gate;
+  SQ_TRY(sd_moe_route_rows_gated(h, W, l.w_router, f32, rlog, sel_e, sel_w, R, l.n_experts, W, l.top, l.route_score,
+                                 l.route_renorm, l.route_renorm_eps, l.route_scale != 0.f ? l.route_scale : 1.f,
+                                 gated_shared ? l.w_shared_gate : nullptr, gated_shared ? 1 : 0, sg, stream));
+  SQ_TRY(sd_moe_experts(h, hb, W, sel_e, sel_w, l.w_gate_up, l.w_down_e, f32, dn, R, l.top, l.n_experts, l.expert_ff, W,
+                        l.expert_scale_input, l.expert_act, base + w.moe, w.moe_bytes, stream));
+  if (l.shared_ff > 0) {
+    const int F = l.shared_ff, n_in = act_inputs(l.shared_act);
+    SQ_TRY(seq_linear(l.w_shared_in, l.w_shared_in_tiled, f32, h, nullptr, W, hb, W, nullptr, proj, (int64_t)n_in * F,
+                      R, n_in * F, W, wide_ws, w.wide_bytes, stream));
+    SQ_TRY(sd_act_rows(proj, n_in > 1 ? proj + F : nullptr, (int64_t)n_in * F, proj, (int64_t)n_in * F,
+                       l.w_shared_down_tiled ? actb : nullptr, F, R, F, l.shared_act, rnd, stream));
+    SQ_TRY(seq_linear(l.w_shared_down, l.w_shared_down_tiled, f32, proj, nullptr, (int64_t)n_in * F, actb, F, nullptr,
+                      ffo, W, R, W, F, wide_ws, w.wide_bytes, stream));
+  }
+  return sd_residual_norm(x, dn, l.top, l.shared_ff > 0 ? ffo : nullptr, gated_shared ? sg : nullptr, 1,
+                          l.post_norm2_w, next_add, next_norm, f32, eps, x_copy, h, hb, R, W, stream);
+}
 }  // namespace
 
 extern "C" int sd_seq_model_forward(sd_seq_model* m, const sd_seq_batch* b, void* workspace,
@@ -1330,7 +1504,7 @@ extern "C" int sd_seq_model_forward(sd_seq_model* m, const sd_seq_batch* b, void
   bf16_t* houtb = (bf16_t*)(base + w.houtb);
   void* wide_ws = base + w.wide;
 
-  const bool hashed = d.bigram || (d.embed_scale != 0.f && d.embed_scale != 1.f) || m->layers[0].block == SD_BLOCK_POSTNORM;
+  const bool hashed = d.bigram || (d.embed_scale != 0.f && d.embed_scale != 1.f) || m->layers[0].block != SD_BLOCK_GATED;
   if (hashed) {
     SD_REQUIRE(!d.bigram || b->prev_tokens, SD_ERR_INVALID, "sd_seq_model_forward: a bigram table needs prev_tokens");
     SQ_TRY(sd_embed_hashed(b->tokens, b->prev_tokens, d.embed, d.bigram, f32, d.embed_scale != 0.f ? d.embed_scale : 1.f,
@@ -1343,6 +1517,14 @@ extern "C" int sd_seq_model_forward(sd_seq_model* m, const sd_seq_batch* b, void
 
   for (int li = 0; li < d.n_layers; ++li) {
     const sd_seq_layer& l = m->layers[li];
+    if (l.block == SD_BLOCK_SANDWICH) {
+      if (li == 0)   // the first layer's input: what is added before it, then its norm
+        SQ_TRY(sd_residual_norm(x, nullptr, 0, nullptr, nullptr, 0, nullptr, l.pre_add, l.norm_w, f32, d.norm_eps,
+                                nullptr, h, hb, R, W, stream));
+      SQ_TRY(sandwich_layer(*m, l, li + 1 < d.n_layers ? &m->layers[li + 1] : nullptr, *b, base, w,
+                            b->layer_out ? b->layer_out + (size_t)li * R * W : nullptr, stream));
+      continue;
+    }
     if (l.block == SD_BLOCK_POSTNORM) {
       SQ_TRY(postnorm_layer(*m, l, *b, base, w, stream));
       if (b->layer_out) {
@@ -1353,7 +1535,7 @@ extern "C" int sd_seq_model_forward(sd_seq_model* m, const sd_seq_batch* b, void
       }
       continue;
     }
-    SD_REQUIRE(li == 0 || m->layers[li - 1].block != SD_BLOCK_POSTNORM, SD_ERR_UNSUPPORTED,
+    SD_REQUIRE(li == 0 || m->layers[li - 1].block == SD_BLOCK_GATED, SD_ERR_UNSUPPORTED,
                "sd_seq_model_forward: a gated layer after a layer normed on its output is not provided");
     const InCols c = in_cols(l, W);
     const int64_t ld = c.total;

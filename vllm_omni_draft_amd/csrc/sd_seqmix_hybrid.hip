@@ -148,6 +148,9 @@ template <> struct Piece<float> {
   }
 };
 
+// A score capped smoothly at +-cap (cap <= 0: as it is).
+__device__ __forceinline__ float cap_score(float s, float cap) { return cap > 0.f ? cap * tanhf(s / cap) : s; }
+
 // s[hq] += q[hq] . k over n channels, ascending (kr and qs point at the first of them; a head's
 // query is q_stride floats from the next).  vec: rows are 16-byte aligned and n a multiple of
 // the piece size; then up to kLoads pieces are asked for before the first is used.
@@ -201,7 +204,8 @@ __global__ __launch_bounds__(256) void window_softmax_attn_kernel(
     int v_row, const int32_t* __restrict__ row_pos, const int32_t* __restrict__ row_slot,
     const int32_t* __restrict__ block_tables, int max_blocks, int page, int H, int G, int dk, int dv, int window,
     int keep_first, float scale, float* __restrict__ out, bf16_t* __restrict__ out_b, int n_hgroups, int n_splits,
-    float* __restrict__ part_acc, float* __restrict__ part_ml) {
+    float* __restrict__ part_acc, float* __restrict__ part_ml, int chunk, float softcap,
+    const float* __restrict__ sinks) {
   extern __shared__ float lds[];
   constexpr int nthr = 256, nw = 4, PARTS = nthr / KT, KW = KT / 64;
   unsigned long long* vat = reinterpret_cast<unsigned long long*>(lds);  // [KT] cache row of the key
@@ -221,10 +225,14 @@ __global__ __launch_bounds__(256) void window_softmax_attn_kernel(
   const int32_t* tbl = block_tables + (size_t)row_slot[r] * max_blocks;
   for (int c = tid; c < nh * dk; c += nthr) qs[c] = q[(size_t)r * ldq + (size_t)h0 * dk + c];
   if (tid < NH) {
-    m_run[tid] = -INFINITY;
-    l_run[tid] = 0.f;
+    // (a sink is one more term exp(sink) of the denominator, with no key and no value: the first
+    // tile's workgroup starts its running maximum and sum from it)
+    const bool sunk = sinks && split == 0 && tid < nh;
+    m_run[tid] = sunk ? sinks[h0 + tid] : -INFINITY;
+    l_run[tid] = sunk ? 1.f : 0.f;
   }
-  const int t_first = i - window + 1 > 0 ? i - window + 1 : 0;
+  int t_first = i - window + 1 > 0 ? i - window + 1 : 0;
+  if (chunk > 0 && i - i % chunk > t_first) t_first = i - i % chunk;   // keys of the row's own chunk only
   const int n_kept = keep_first < t_first ? keep_first : t_first;   // kept tokens that left the window
   const int total = n_kept + (i - t_first + 1);
   const int key_lo = n_splits > 1 ? split * KT : 0;
@@ -258,7 +266,7 @@ __global__ __launch_bounds__(256) void window_softmax_attn_kernel(
       if constexpr (PARTS == 1) {
 #pragma unroll
         for (int hq = 0; hq < NH; ++hq)
-          if (hq < nh) wt[hq * KT + key] = idx < key_hi ? s[hq] * scale : -INFINITY;
+          if (hq < nh) wt[hq * KT + key] = idx < key_hi ? cap_score(s[hq] * scale, softcap) : -INFINITY;
       } else {
 #pragma unroll
         for (int hq = 0; hq < NH; ++hq)
@@ -271,7 +279,7 @@ __global__ __launch_bounds__(256) void window_softmax_attn_kernel(
               float sum = ps[hq * KT + key];
 #pragma unroll
               for (int pp = 1; pp < PARTS; ++pp) sum += ps[(pp * NH + hq) * KT + key];
-              wt[hq * KT + key] = idx < key_hi ? sum * scale : -INFINITY;
+              wt[hq * KT + key] = idx < key_hi ? cap_score(sum * scale, softcap) : -INFINITY;
             }
         }
       }
@@ -349,6 +357,7 @@ __global__ __launch_bounds__(256) void window_softmax_attn_kernel(
       for (int m = 0; m < NC; ++m)
         if (lane + 64 * m < dv) red[wave * dv + lane + 64 * m] = acc[hq][m];
       __syncthreads();
+      // (no key and no sink: a row past its own keys, which a cut launch's merge skips)
       const float inv = n_splits > 1 ? 1.f : 1.f / l_run[hq];
       for (int c = tid; c < dv; c += nthr) {
         float o = red[c];
@@ -405,12 +414,12 @@ void launch_softmax_nc(dim3 grid, int kt, size_t lds, hipStream_t st, int nc, co
                        const void* kc, const void* vc, int v_row, const int32_t* row_pos, const int32_t* row_slot,
                        const int32_t* bt, int max_blocks, int page, int H, int G, int dk, int dv, int window,
                        int keep_first, float scale, float* out, bf16_t* out_b, int n_hgroups, int n_splits,
-                       float* part_acc, float* part_ml) {
+                       float* part_acc, float* part_ml, int chunk, float softcap, const float* sinks) {
 #define SD_GO2(NC, KT)                                                                                               \
   window_softmax_attn_kernel<T, NH, NC, KT><<<grid, 256, lds, st>>>(q, ldq, (const T*)kc, (const T*)vc, v_row, row_pos, \
                                                                     row_slot, bt, max_blocks, page, H, G, dk, dv,       \
                                                                     window, keep_first, scale, out, out_b, n_hgroups,   \
-                                                                    n_splits, part_acc, part_ml)
+                                                                    n_splits, part_acc, part_ml, chunk, softcap, sinks)
 #define SD_GO(NC)                                          \
   do {                                                     \
     if constexpr (NH <= 4) {                               \
@@ -455,7 +464,7 @@ __global__ __launch_bounds__(256) void latent_prep_kernel(
     T* __restrict__ k_cache) {
   __shared__ float red[4];
   const int r = blockIdx.x;
-  if (blockIdx.y == 0) {
+  if (blockIdx.y == 0 && q_lat) {
     norm_in_place<T>(q_lat + (size_t)r * ld, q_w, q_rank, eps, round, q_copy ? q_copy + (size_t)r * ld_copy : nullptr, red);
     return;
   }
@@ -506,6 +515,82 @@ __global__ __launch_bounds__(256) void qk_norm_append_kernel(
   for (int c = threadIdx.x; c < G * dv; c += blockDim.x) {
     const int g = c / dv;
     st_f(v_cache + (((size_t)pg * G + g) * page + pos % page) * dv + c % dv, vr[c]);
+  }
+}
+
+// Attention whose q and k are normed per head with one weight [dk] shared by the heads, per row.
+// Workgroup (r, 0): the H query heads in place, a wave per head.  Workgroup (r, 1): the G key
+// heads in place, then the key and value rows appended.
+template <typename T>
+__device__ __forceinline__ void norm_heads_in_place(float* __restrict__ v, int heads, int dk, const T* __restrict__ w,
+                                                    float eps) {
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, nw = blockDim.x >> 6;
+  for (int h = wave; h < heads; h += nw) {
+    float* x = v + (size_t)h * dk;
+    float ss = 0.f;
+    for (int c = lane; c < dk; c += 64) ss = fmaf(x[c], x[c], ss);
+    ss = wave_sum(ss);
+    const float rstd = 1.f / sqrtf(ss / (float)dk + eps);
+    for (int c = lane; c < dk; c += 64) x[c] = x[c] * rstd * ld_f(w + c);
+  }
+}
+template <typename T>
+__global__ __launch_bounds__(256) void qk_head_norm_append_kernel(
+    float* __restrict__ q, int H, const T* __restrict__ q_w, float* __restrict__ k, int G, int dk,
+    const T* __restrict__ k_w, const float* __restrict__ v, int dv, int64_t ld, float eps,
+    const int32_t* __restrict__ row_pos, const int32_t* __restrict__ row_slot,
+    const int32_t* __restrict__ block_tables, int max_blocks, int page, T* __restrict__ k_cache,
+    T* __restrict__ v_cache) {
+  const int r = blockIdx.x;
+  if (blockIdx.y == 0) {
+    norm_heads_in_place<T>(q + (size_t)r * ld, H, dk, q_w, eps);
+    return;
+  }
+  float* kr = k + (size_t)r * ld;
+  norm_heads_in_place<T>(kr, G, dk, k_w, eps);
+  __syncthreads();
+  const int pos = row_pos[r];
+  const int pg = block_tables[(size_t)row_slot[r] * max_blocks + pos / page];
+  for (int c = threadIdx.x; c < G * dk; c += blockDim.x) {
+    const int g = c / dk;
+    st_f(k_cache + (((size_t)pg * G + g) * page + pos % page) * dk + c % dk, kr[c]);
+  }
+  const float* vr = v + (size_t)r * ld;
+  for (int c = threadIdx.x; c < G * dv; c += blockDim.x) {
+    const int g = c / dv;
+    st_f(v_cache + (((size_t)pg * G + g) * page + pos % page) * dv + c % dv, vr[c]);
+  }
+}
+
+// y[r, h, :] *= sigmoid(z[r, h]): one gate per (row, head).  y_b (or nullptr): the result as bf16.
+__global__ void head_gate_kernel(float* __restrict__ y, int64_t ldy, const float* __restrict__ z, int64_t ldz,
+                                 bf16_t* __restrict__ y_b, int64_t ldyb, int H, int dv, int round) {
+  const int r = blockIdx.x;
+  for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < H * dv; c += gridDim.y * blockDim.x) {
+    const float o = maybe_round(y[(size_t)r * ldy + c] * sigmoid_f(z[(size_t)r * ldz + c / dv]), round);
+    y[(size_t)r * ldy + c] = o;
+    if (y_b) y_b[(size_t)r * ldyb + c] = (bf16_t)o;
+  }
+}
+
+// A feed-forward's activation, a[r, c]: kind 0 relu(g) u, 1 silu(g) u, 2 relu(g)^2 (no u).
+// out (may be g itself) and out_b (bf16, or nullptr) receive it.
+__global__ void act_rows_kernel(const float* __restrict__ g, const float* __restrict__ u, int64_t ld,
+                                float* __restrict__ out, int64_t ldo, bf16_t* __restrict__ out_b, int64_t ldob, int F,
+                                int kind, int round) {
+  const int r = blockIdx.x;
+  for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < F; c += gridDim.y * blockDim.x) {
+    const float z = g[(size_t)r * ld + c];
+    float a;
+    if (kind == 2) {
+      const float p = fmaxf(z, 0.f);
+      a = p * p;
+    } else {
+      a = (kind == 1 ? silu_f(z) : fmaxf(z, 0.f)) * u[(size_t)r * ld + c];
+    }
+    a = maybe_round(a, round);
+    if (out) out[(size_t)r * ldo + c] = a;
+    if (out_b) out_b[(size_t)r * ldob + c] = (bf16_t)a;
   }
 }
 
@@ -741,13 +826,16 @@ __global__ __launch_bounds__(1024) void moe_route_rows_kernel(const float* __res
                                                              const T* __restrict__ w, float* __restrict__ logits,
                                                              int32_t* __restrict__ sel_e, float* __restrict__ sel_w,
                                                              int E, int K, int top, int score_kind, int renorm,
-                                                             int round) {
+                                                             int round, float renorm_eps, float weight_scale,
+                                                             const T* __restrict__ w_gate, int n_gate,
+                                                             float* __restrict__ gate_out) {
   extern __shared__ float sc[];   // [E]
   const int r = blockIdx.x, wave = threadIdx.x >> 6, lane = threadIdx.x & 63, nw = blockDim.x >> 6;
   const float* xr = x + (size_t)r * ldx;
   constexpr int kU = 8;   // loads of a lane in flight
-  for (int e = wave; e < E; e += nw) {
-    const T* wr = w + (size_t)e * K;
+  // (rows E .. E + n_gate - 1 are further products of the same input: gates computed as the router is)
+  for (int e = wave; e < E + n_gate; e += nw) {
+    const T* wr = e < E ? w + (size_t)e * K : w_gate + (size_t)(e - E) * K;
     float acc = 0.f;
     for (int k0 = 0; k0 < K; k0 += 64 * kU) {
       float xv[kU], wv[kU];
@@ -763,8 +851,12 @@ __global__ __launch_bounds__(1024) void moe_route_rows_kernel(const float* __res
     }
     acc = wave_sum(acc);
     if (lane == 0) {
-      sc[e] = acc;
-      if (logits) logits[(size_t)r * E + e] = acc;
+      if (e < E) {
+        sc[e] = acc;
+        if (logits) logits[(size_t)r * E + e] = acc;
+      } else {
+        gate_out[(size_t)r * n_gate + e - E] = acc;
+      }
     }
   }
   __syncthreads();
@@ -811,8 +903,21 @@ __global__ __launch_bounds__(1024) void moe_route_rows_kernel(const float* __res
     }
     total += best;
   }
-  if (renorm && lane == 0)
-    for (int j = 0; j < top; ++j) sel_w[(size_t)r * top + j] /= total;
+  if (lane == 0 && (renorm || weight_scale != 1.f))
+    for (int j = 0; j < top; ++j) {
+      const float v = sel_w[(size_t)r * top + j];
+      sel_w[(size_t)r * top + j] = (renorm ? v / (total + renorm_eps) : v) * weight_scale;
+    }
+}
+
+// An expert's activation from its (scaled) first product a and, when gated, its second product u:
+// kind 0 silu(a) u; kind 1 relu(a)^2, an expert of two matrices only.
+__device__ __forceinline__ float expert_act(float a, float u, int kind) {
+  if (kind == 1) {
+    const float p = fmaxf(a, 0.f);
+    return p * p;
+  }
+  return silu_f(a) * u;
 }
 
 constexpr int kMoeBM = 32;   // assignment rows per tile of the grouped products
@@ -871,8 +976,9 @@ template <typename T>
 __global__ __launch_bounds__(256) void moe_gate_up_kernel(
     const float* __restrict__ X, int64_t ldx, const int32_t* __restrict__ perm, const int32_t* __restrict__ tiles,
     const int32_t* __restrict__ n_tiles, const float* __restrict__ sel_w, const T* __restrict__ Wgu,
-    float* __restrict__ act, int top, int F, int K, int scale_input, int round) {
+    float* __restrict__ act, int top, int F, int K, int scale_input, int round, int act_kind) {
   constexpr int BM = kMoeBM, BN = 64, BK = 16, TM = 2, TN = 4;
+  const bool gated = act_kind == 0;   // (else Wgu holds one matrix [F, K] per expert)
   if (tiles && (int)blockIdx.y >= n_tiles[0]) return;
   __shared__ float xs[BK][BM + 1];
   __shared__ float wg[BK][BN + 1];
@@ -883,8 +989,8 @@ __global__ __launch_bounds__(256) void moe_gate_up_kernel(
   const int p0 = tiles ? tiles[3 * blockIdx.y + 1] : blockIdx.y, rows = tiles ? tiles[3 * blockIdx.y + 2] : 1;
   const int tid = threadIdx.x, tx = tid % (BN / TN), ty = tid / (BN / TN);
   const int n0 = blockIdx.x * BN;
-  const T* Wg = Wgu + (size_t)e * 2 * F * K;
-  const T* Wu = Wg + (size_t)F * K;
+  const T* Wg = Wgu + (size_t)e * (gated ? 2 : 1) * F * K;
+  const T* Wu = gated ? Wg + (size_t)F * K : Wg;
   if (tid < BM) arow[tid] = tid < rows ? (tiles ? perm[p0 + tid] : p0) : -1;
   __syncthreads();
   float ag[TM][TN], au[TM][TN];
@@ -902,7 +1008,7 @@ __global__ __launch_bounds__(256) void moe_gate_up_kernel(
       const int n = idx / BK, kk = idx % BK;
       const bool in = n0 + n < F && k0 + kk < K;
       wg[kk][n] = in ? ld_f(Wg + (size_t)(n0 + n) * K + k0 + kk) : 0.f;
-      wu[kk][n] = in ? ld_f(Wu + (size_t)(n0 + n) * K + k0 + kk) : 0.f;
+      wu[kk][n] = in && gated ? ld_f(Wu + (size_t)(n0 + n) * K + k0 + kk) : 0.f;
     }
     __syncthreads();
 #pragma unroll
@@ -933,7 +1039,7 @@ __global__ __launch_bounds__(256) void moe_gate_up_kernel(
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
       const int n = n0 + tx * TN + j;
-      if (n < F) act[(size_t)a * F + n] = maybe_round(silu_f(s * ag[i][j]) * (s * au[i][j]), round);
+      if (n < F) act[(size_t)a * F + n] = maybe_round(expert_act(s * ag[i][j], s * au[i][j], act_kind), round);
     }
   }
 }
@@ -1011,7 +1117,7 @@ __device__ __forceinline__ f32x4 mfma16(bf16x8 a, bf16x8 b, f32x4 c) {
 
 // act[a, n] (bf16) = silu(s * gate) * (s * up); a wave owns 32 columns of gate and of up.  Xb (or
 // nullptr): the rows of X as bf16 already.
-template <int MT, int KC>
+template <int MT, int KC, bool GATED>
 __global__ __launch_bounds__(256) void moe_gate_up_mfma_kernel(
     const float* __restrict__ X, const bf16_t* __restrict__ Xb, int64_t ldx, const int32_t* __restrict__ perm,
     const int32_t* __restrict__ tiles, const int32_t* __restrict__ n_tiles, const float* __restrict__ sel_w,
@@ -1025,10 +1131,11 @@ __global__ __launch_bounds__(256) void moe_gate_up_mfma_kernel(
   const int p0 = tiles ? tiles[3 * blockIdx.y + 1] : blockIdx.y, rows = tiles ? tiles[3 * blockIdx.y + 2] : 1;
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, lr = lane & 15, kq = lane >> 4;
   const int n0 = blockIdx.x * 128 + wave * 32 + lr, n1 = n0 + 16;
-  const bf16_t* wg0 = Wgu + ((size_t)e * 2 * F + (n0 < F ? n0 : F - 1)) * K + 8 * kq;
-  const bf16_t* wg1 = Wgu + ((size_t)e * 2 * F + (n1 < F ? n1 : F - 1)) * K + 8 * kq;
-  const bf16_t* wu0 = wg0 + (size_t)F * K;
-  const bf16_t* wu1 = wg1 + (size_t)F * K;
+  constexpr int NM = GATED ? 2 : 1;   // matrices of an expert in Wgu
+  const bf16_t* wg0 = Wgu + ((size_t)e * NM * F + (n0 < F ? n0 : F - 1)) * K + 8 * kq;
+  const bf16_t* wg1 = Wgu + ((size_t)e * NM * F + (n1 < F ? n1 : F - 1)) * K + 8 * kq;
+  const bf16_t* wu0 = GATED ? wg0 + (size_t)F * K : wg0;
+  const bf16_t* wu1 = GATED ? wg1 + (size_t)F * K : wg1;
   if (tid < BM) arow[tid] = tid < rows ? (tiles ? perm[p0 + tid] : p0) : -1;
   f32x4 ag[MT][2], au[MT][2];
 #pragma unroll
@@ -1062,16 +1169,21 @@ __global__ __launch_bounds__(256) void moe_gate_up_mfma_kernel(
     for (int k0 = 0; k0 < kc; k0 += 32) {
       const bf16x8 fg0 = *reinterpret_cast<const bf16x8*>(wg0 + kc0 + k0);
       const bf16x8 fg1 = *reinterpret_cast<const bf16x8*>(wg1 + kc0 + k0);
-      const bf16x8 fu0 = *reinterpret_cast<const bf16x8*>(wu0 + kc0 + k0);
-      const bf16x8 fu1 = *reinterpret_cast<const bf16x8*>(wu1 + kc0 + k0);
+      bf16x8 fu0 = fg0, fu1 = fg1;
+      if constexpr (GATED) {
+        fu0 = *reinterpret_cast<const bf16x8*>(wu0 + kc0 + k0);
+        fu1 = *reinterpret_cast<const bf16x8*>(wu1 + kc0 + k0);
+      }
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) {
         if (mt < m_tiles) {
           const bf16x8 a = *reinterpret_cast<const bf16x8*>(xs + (16 * mt + lr) * LD + k0 + 8 * kq);
           ag[mt][0] = mfma16(a, fg0, ag[mt][0]);
           ag[mt][1] = mfma16(a, fg1, ag[mt][1]);
-          au[mt][0] = mfma16(a, fu0, au[mt][0]);
-          au[mt][1] = mfma16(a, fu1, au[mt][1]);
+          if constexpr (GATED) {
+            au[mt][0] = mfma16(a, fu0, au[mt][0]);
+            au[mt][1] = mfma16(a, fu1, au[mt][1]);
+          }
         }
       }
     }
@@ -1083,8 +1195,8 @@ __global__ __launch_bounds__(256) void moe_gate_up_mfma_kernel(
       const int a = arow[mt * 16 + 4 * kq + i];
       if (a < 0) continue;
       const float sc = scale_input ? sel_w[a] : 1.f;
-      if (n0 < F) act[(size_t)a * F + n0] = (bf16_t)(silu_f(sc * ag[mt][0][i]) * (sc * au[mt][0][i]));
-      if (n1 < F) act[(size_t)a * F + n1] = (bf16_t)(silu_f(sc * ag[mt][1][i]) * (sc * au[mt][1][i]));
+      if (n0 < F) act[(size_t)a * F + n0] = (bf16_t)expert_act(sc * ag[mt][0][i], sc * au[mt][0][i], GATED ? 0 : 1);
+      if (n1 < F) act[(size_t)a * F + n1] = (bf16_t)expert_act(sc * ag[mt][1][i], sc * au[mt][1][i], GATED ? 0 : 1);
     }
 }
 
@@ -1152,6 +1264,7 @@ __global__ __launch_bounds__(256) void moe_down_mfma_kernel(
 // loads asked for before the first is used), then a butterfly sum.
 constexpr int kGemvMaxK = 8192;
 // act[a, n] (bf16) = silu(s * gate_e[n] . x) * (s * up_e[n] . x); wave: two columns, gate and up.
+template <bool GATED>
 __global__ __launch_bounds__(256) void moe_gemv_gate_up_kernel(
     const float* __restrict__ X, int64_t ldx, const int32_t* __restrict__ sel_e, const float* __restrict__ sel_w,
     const bf16_t* __restrict__ Wgu, bf16_t* __restrict__ act, int top, int F, int K, int scale_input) {
@@ -1163,8 +1276,9 @@ __global__ __launch_bounds__(256) void moe_gemv_gate_up_kernel(
   const int n0 = blockIdx.x * 8 + wave * 2;
   if (n0 >= F) return;
   const int n1 = n0 + 1 < F ? n0 + 1 : n0;
-  const bf16_t* wg = Wgu + (size_t)e * 2 * F * K;
-  const bf16_t* wu = wg + (size_t)F * K;
+  // (not gated: an expert is one matrix [F, K]; the "up" rows alias the first, their sums go unused)
+  const bf16_t* wg = Wgu + (size_t)e * (GATED ? 2 : 1) * F * K;
+  const bf16_t* wu = GATED ? wg + (size_t)F * K : wg;
   const bf16_t* rows[4] = {wg + (size_t)n0 * K, wu + (size_t)n0 * K, wg + (size_t)n1 * K, wu + (size_t)n1 * K};
   float acc[4] = {0.f, 0.f, 0.f, 0.f};
   for (int k0 = lane * 8; k0 < K; k0 += 4 * 512) {
@@ -1192,8 +1306,8 @@ __global__ __launch_bounds__(256) void moe_gemv_gate_up_kernel(
   for (int j = 0; j < 4; ++j) acc[j] = wave_sum(acc[j]);
   if (lane == 0) {
     const float sc = scale_input ? sel_w[a] : 1.f;
-    act[(size_t)a * F + n0] = (bf16_t)(silu_f(sc * acc[0]) * (sc * acc[1]));
-    if (n0 + 1 < F) act[(size_t)a * F + n0 + 1] = (bf16_t)(silu_f(sc * acc[2]) * (sc * acc[3]));
+    act[(size_t)a * F + n0] = (bf16_t)expert_act(sc * acc[0], sc * acc[1], GATED ? 0 : 1);
+    if (n0 + 1 < F) act[(size_t)a * F + n0 + 1] = (bf16_t)expert_act(sc * acc[2], sc * acc[3], GATED ? 0 : 1);
   }
 }
 
@@ -1288,6 +1402,54 @@ __global__ void postnorm_residual_kernel(float* __restrict__ x, const float* __r
   }
 }
 
+// A layer normed before and after its sublayers, per row, in one launch:
+//   t = the sum of the row's n_a rows of a (+ sigmoid(b_gate[r]) * b[r]);  x += rms_norm(t) * w_post
+// (a == nullptr: no update); x_copy (or nullptr) receives the row as it is then; x += add (a
+// vector [W], or nullptr); unless w_next == nullptr, h = rms_norm(x) * w_next, the input of the
+// sublayer that follows (h_b: the same as bf16).  The row is held in LDS between the steps.
+template <typename T>
+__global__ __launch_bounds__(256) void residual_norm_kernel(
+    float* __restrict__ x, const float* __restrict__ a, int n_a, const float* __restrict__ b,
+    const float* __restrict__ b_gate, int64_t ldg, const T* __restrict__ w_post, const T* __restrict__ add,
+    const T* __restrict__ w_next, float eps, float* __restrict__ x_copy, float* __restrict__ h,
+    bf16_t* __restrict__ h_b, int W, int round) {
+  extern __shared__ float row[];   // [W]
+  __shared__ float red[4];
+  const int r = blockIdx.x;
+  float rstd = 0.f;
+  if (a) {
+    const float gate = b ? (b_gate ? sigmoid_f(b_gate[(size_t)r * ldg]) : 1.f) : 0.f;
+    float ss = 0.f;
+    for (int c = threadIdx.x; c < W; c += blockDim.x) {
+      float v = a[((size_t)r * n_a) * W + c];
+      for (int j = 1; j < n_a; ++j) v += a[((size_t)r * n_a + j) * W + c];
+      if (b) v += gate * b[(size_t)r * W + c];
+      row[c] = v;
+      ss = fmaf(v, v, ss);
+    }
+    ss = block_sum(ss, red);
+    rstd = 1.f / sqrtf(ss / (float)W + eps);
+  }
+  float ss2 = 0.f;
+  for (int c = threadIdx.x; c < W; c += blockDim.x) {
+    float xn = x[(size_t)r * W + c];
+    if (a) xn += row[c] * rstd * ld_f(w_post + c);
+    if (x_copy) x_copy[(size_t)r * W + c] = xn;
+    if (add) xn += ld_f(add + c);
+    if (a || add) x[(size_t)r * W + c] = xn;
+    row[c] = xn;
+    ss2 = fmaf(xn, xn, ss2);
+  }
+  if (!w_next) return;
+  ss2 = block_sum(ss2, red);
+  const float rstd2 = 1.f / sqrtf(ss2 / (float)W + eps);
+  for (int c = threadIdx.x; c < W; c += blockDim.x) {
+    const float v = maybe_round(row[c] * rstd2 * ld_f(w_next + c), round);
+    if (h) h[(size_t)r * W + c] = v;
+    if (h_b) h_b[(size_t)r * W + c] = (bf16_t)v;
+  }
+}
+
 __global__ void scale_rows_kernel(float* __restrict__ x, int64_t ld, float s, int n_cols) {
   const int r = blockIdx.x;
   for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < n_cols; c += gridDim.y * blockDim.x)
@@ -1359,14 +1521,14 @@ extern "C" int sd_latent_prep(float* q_latent, int q_rank, const void* q_norm_w,
                               float eps, int rot_dims, int rot_layout, const double* inv_freq, float mag, void* k_cache,
                               const int32_t* row_pos, const int32_t* row_slot, const int32_t* block_tables,
                               int max_blocks, int page, int n_rows, sd_stream_t stream) {
-  SD_REQUIRE(q_latent && q_norm_w && kv && kv_norm_w && k_cache && row_pos && row_slot && block_tables, SD_ERR_INVALID,
+  SD_REQUIRE((!q_latent || q_norm_w) && kv && kv_norm_w && k_cache && row_pos && row_slot && block_tables, SD_ERR_INVALID,
              "sd_latent_prep: null argument");
-  SD_REQUIRE(n_rows >= 1 && q_rank >= 1 && kv_rank >= 1 && rot_dim >= 0 && page >= 1 && max_blocks >= 1, SD_ERR_INVALID,
+  SD_REQUIRE(n_rows >= 1 && (!q_latent || q_rank >= 1) && kv_rank >= 1 && rot_dim >= 0 && page >= 1 && max_blocks >= 1, SD_ERR_INVALID,
              "sd_latent_prep: bad shape");
   SD_REQUIRE(rot_dims >= 0 && rot_dims % 2 == 0 && rot_dims <= rot_dim && (rot_dims == 0 || inv_freq), SD_ERR_INVALID,
              "sd_latent_prep: rot_dims %d must be even, at most rot_dim %d, with a frequency table", rot_dims, rot_dim);
   hipStream_t st = (hipStream_t)stream;
-  dim3 grid(n_rows, 2);
+  dim3 grid(n_rows, q_latent ? 2 : 1);   // (queries that come straight from the input have no latent to norm)
   if (w_f32)
     latent_prep_kernel<float><<<grid, 256, 0, st>>>(q_latent, q_rank, (const float*)q_norm_w, (bf16_t*)q_bf16, ld_q_bf16,
                                                     kv, kv_rank, rot_dim, (const float*)kv_norm_w, ld, eps, 0, rot_dims,
@@ -1403,6 +1565,56 @@ extern "C" int sd_qk_norm_append(float* q, int n_q, const void* q_norm_w, float*
   return SD_OK;
 }
 
+extern "C" int sd_qk_head_norm_append(float* q, int H, const void* q_norm_w, float* k, int G, int dk,
+                                      const void* k_norm_w, const float* v, int dv, int64_t ld, int w_f32, float eps,
+                                      void* k_cache, void* v_cache, const int32_t* row_pos, const int32_t* row_slot,
+                                      const int32_t* block_tables, int max_blocks, int page, int n_rows,
+                                      sd_stream_t stream) {
+  SD_REQUIRE(q && q_norm_w && k && k_norm_w && v && k_cache && v_cache && row_pos && row_slot && block_tables,
+             SD_ERR_INVALID, "sd_qk_head_norm_append: null argument");
+  SD_REQUIRE(n_rows >= 1 && H >= 1 && G >= 1 && dk >= 1 && dv >= 1 && page >= 1 && max_blocks >= 1, SD_ERR_INVALID,
+             "sd_qk_head_norm_append: bad shape");
+  hipStream_t st = (hipStream_t)stream;
+  dim3 grid(n_rows, 2);
+  if (w_f32)
+    qk_head_norm_append_kernel<float><<<grid, 256, 0, st>>>(q, H, (const float*)q_norm_w, k, G, dk,
+                                                            (const float*)k_norm_w, v, dv, ld, eps, row_pos, row_slot,
+                                                            block_tables, max_blocks, page, (float*)k_cache,
+                                                            (float*)v_cache);
+  else
+    qk_head_norm_append_kernel<bf16_t><<<grid, 256, 0, st>>>(q, H, (const bf16_t*)q_norm_w, k, G, dk,
+                                                             (const bf16_t*)k_norm_w, v, dv, ld, eps, row_pos, row_slot,
+                                                             block_tables, max_blocks, page, (bf16_t*)k_cache,
+                                                             (bf16_t*)v_cache);
+  SD_CHECK_LAUNCH("sd_qk_head_norm_append");
+  return SD_OK;
+}
+
+extern "C" int sd_head_gate_rows(float* y, int64_t ldy, const float* z, int64_t ldz, void* y_bf16, int64_t ldyb,
+                                 int n_rows, int H, int dv, int round_bf16_out, sd_stream_t stream) {
+  SD_REQUIRE(y && z && n_rows >= 1 && H >= 1 && dv >= 1 && ldy >= (int64_t)H * dv && ldz >= H, SD_ERR_INVALID,
+             "sd_head_gate_rows: bad argument");
+  int by = (H * dv + 255) / 256;
+  if (by > 32) by = 32;
+  head_gate_kernel<<<dim3(n_rows, by), 256, 0, (hipStream_t)stream>>>(y, ldy, z, ldz, (bf16_t*)y_bf16, ldyb, H, dv,
+                                                                      round_bf16_out);
+  SD_CHECK_LAUNCH("sd_head_gate_rows");
+  return SD_OK;
+}
+
+extern "C" int sd_act_rows(const float* gate, const float* up, int64_t ld, float* out, int64_t ldo, void* out_bf16,
+                           int64_t ldob, int n_rows, int F, int act_kind, int round_bf16_out, sd_stream_t stream) {
+  SD_REQUIRE(gate && (out || out_bf16) && n_rows >= 1 && F >= 1 && ld >= F, SD_ERR_INVALID, "sd_act_rows: bad argument");
+  SD_REQUIRE(act_kind >= 0 && act_kind <= 2 && (act_kind == 2 || up), SD_ERR_INVALID,
+             "sd_act_rows: activation %d unknown, or a gated one without its second input", act_kind);
+  int by = (F + 255) / 256;
+  if (by > 64) by = 64;
+  act_rows_kernel<<<dim3(n_rows, by), 256, 0, (hipStream_t)stream>>>(gate, up, ld, out, ldo, (bf16_t*)out_bf16, ldob, F,
+                                                                     act_kind, round_bf16_out);
+  SD_CHECK_LAUNCH("sd_act_rows");
+  return SD_OK;
+}
+
 extern "C" int sd_cache_append(const float* k, int64_t ldk, const float* v, int64_t ldv, void* k_cache, void* v_cache,
                                int cache_f32, const int32_t* row_pos, const int32_t* row_slot,
                                const int32_t* block_tables, int max_blocks, int page, int n_rows, int G, int dk, int dv,
@@ -1422,29 +1634,31 @@ extern "C" int sd_cache_append(const float* k, int64_t ldk, const float* v, int6
   return SD_OK;
 }
 
-extern "C" size_t sd_window_softmax_attention_scratch_bytes(int n_rows, int H, int dv, int window, int keep_first,
-                                                             int max_ctx) {
+extern "C" size_t sd_masked_softmax_attention_scratch_bytes(int n_rows, int H, int dv, int window, int keep_first,
+                                                             int chunk, int max_ctx) {
   if (n_rows < 1 || n_rows > kSplitRows || H < 1 || dv < 1 || window < 1) return 0;
-  long long max_keys = (long long)window + (keep_first > 0 ? keep_first : 0);
+  long long max_keys = (long long)(chunk > 0 && chunk < window ? chunk : window) + (keep_first > 0 ? keep_first : 0);
   if (max_keys > max_ctx) max_keys = max_ctx;
   const int splits = (int)((max_keys + kSplitKeys - 1) / kSplitKeys);
   return splits > 1 ? (size_t)splits * n_rows * H * (dv + 2) * sizeof(float) : 0;
 }
 
-extern "C" int sd_window_softmax_attention(const float* q, int64_t ldq, const void* k_cache, const void* v_cache,
+extern "C" int sd_masked_softmax_attention(const float* q, int64_t ldq, const void* k_cache, const void* v_cache,
                                            int cache_f32, const int32_t* row_pos, const int32_t* row_slot,
                                            const int32_t* block_tables, int max_blocks, int page, int n_rows, int H,
-                                           int G, int dk, int dv, int window, int keep_first, float scale, float* out,
-                                           void* out_bf16, void* scratch, size_t scratch_bytes, sd_stream_t stream) {
+                                           int G, int dk, int dv, int window, int keep_first, int chunk, float scale,
+                                           float softcap, const float* sinks, float* out, void* out_bf16,
+                                           void* scratch, size_t scratch_bytes, sd_stream_t stream) {
   SD_REQUIRE(q && k_cache && row_pos && row_slot && block_tables && out, SD_ERR_INVALID,
-             "sd_window_softmax_attention: null argument");
-  SD_REQUIRE(n_rows >= 1 && H >= 1 && G >= 1 && H % G == 0 && dk >= 1 && window >= 1 && keep_first >= 0 && page >= 1,
-             SD_ERR_INVALID, "sd_window_softmax_attention: bad shape");
+             "sd_masked_softmax_attention: null argument");
+  SD_REQUIRE(n_rows >= 1 && H >= 1 && G >= 1 && H % G == 0 && dk >= 1 && window >= 1 && keep_first >= 0 && page >= 1 &&
+                 chunk >= 0 && softcap >= 0.f,
+             SD_ERR_INVALID, "sd_masked_softmax_attention: bad shape");
   SD_REQUIRE(dv >= 1 && dv <= 512 && (v_cache || dv <= dk), SD_ERR_UNSUPPORTED,
-             "sd_window_softmax_attention: value size %d outside 1..512 (or above the key row it is part of)", dv);
+             "sd_masked_softmax_attention: value size %d outside 1..512 (or above the key row it is part of)", dv);
   hipStream_t st = (hipStream_t)stream;
   const int qh = H / G;
-  const size_t need = sd_window_softmax_attention_scratch_bytes(n_rows, H, dv, window, keep_first, max_blocks * page);
+  const size_t need = sd_masked_softmax_attention_scratch_bytes(n_rows, H, dv, window, keep_first, chunk, max_blocks * page);
   const bool split = need > 0 && scratch && scratch_bytes >= need && sd_aligned16(scratch);
   const int n_splits = split ? (int)(need / ((size_t)n_rows * H * (dv + 2) * sizeof(float))) : 1;
   const int kt = split ? kSplitKeys : 256;   // keys per tile
@@ -1456,7 +1670,7 @@ extern "C" int sd_window_softmax_attention(const float* q, int64_t ldq, const vo
   const size_t lds = sizeof(unsigned long long) * kt +
                      sizeof(float) * ((size_t)NH * kt + (size_t)NH * dk + 3 * (size_t)NH + (size_t)4 * dv +
                                       (kt < 256 ? (size_t)(256 / kt) * NH * kt : 0));
-  SD_REQUIRE(lds <= 64 * 1024, SD_ERR_UNSUPPORTED, "sd_window_softmax_attention: dim %d / vdim %d need %zu bytes of LDS",
+  SD_REQUIRE(lds <= 64 * 1024, SD_ERR_UNSUPPORTED, "sd_masked_softmax_attention: dim %d / vdim %d need %zu bytes of LDS",
              dk, dv, lds);
   const void* vc = v_cache ? v_cache : k_cache;
   const int v_row = v_cache ? dv : dk;
@@ -1466,7 +1680,7 @@ extern "C" int sd_window_softmax_attention(const float* q, int64_t ldq, const vo
 #define SD_NH(T, N)                                                                                                  \
   launch_softmax_nc<T, N>(grid, kt, lds, st, nc, q, ldq, k_cache, vc, v_row, row_pos, row_slot, block_tables,      \
                           max_blocks, page, H, G, dk, dv, window, keep_first, scale, out, (bf16_t*)out_bf16, n_hgroups, \
-                          n_splits, part_acc, part_ml)
+                          n_splits, part_acc, part_ml, chunk, softcap, sinks)
 #define SD_T(T)                      \
   do {                               \
     if (NH == 1) SD_NH(T, 1);        \
@@ -1478,13 +1692,28 @@ extern "C" int sd_window_softmax_attention(const float* q, int64_t ldq, const vo
   else SD_T(bf16_t);
 #undef SD_T
 #undef SD_NH
-  SD_CHECK_LAUNCH("sd_window_softmax_attention");
+  SD_CHECK_LAUNCH("sd_masked_softmax_attention");
   if (split) {
     softmax_merge_kernel<<<dim3(n_rows, H), dv <= 64 ? 64 : (dv <= 128 ? 128 : 256), 0, st>>>(
         part_acc, part_ml, n_splits, out, (bf16_t*)out_bf16, H, dv);
-    SD_CHECK_LAUNCH("sd_window_softmax_attention (merge)");
+    SD_CHECK_LAUNCH("sd_masked_softmax_attention (merge)");
   }
   return SD_OK;
+}
+
+extern "C" size_t sd_window_softmax_attention_scratch_bytes(int n_rows, int H, int dv, int window, int keep_first,
+                                                             int max_ctx) {
+  return sd_masked_softmax_attention_scratch_bytes(n_rows, H, dv, window, keep_first, 0, max_ctx);
+}
+
+extern "C" int sd_window_softmax_attention(const float* q, int64_t ldq, const void* k_cache, const void* v_cache,
+                                           int cache_f32, const int32_t* row_pos, const int32_t* row_slot,
+                                           const int32_t* block_tables, int max_blocks, int page, int n_rows, int H,
+                                           int G, int dk, int dv, int window, int keep_first, float scale, float* out,
+                                           void* out_bf16, void* scratch, size_t scratch_bytes, sd_stream_t stream) {
+  return sd_masked_softmax_attention(q, ldq, k_cache, v_cache, cache_f32, row_pos, row_slot, block_tables, max_blocks,
+                                     page, n_rows, H, G, dk, dv, window, keep_first, 0, scale, 0.f, nullptr, out,
+                                     out_bf16, scratch, scratch_bytes, stream);
 }
 
 extern "C" int sd_causal_conv_rows(const float* x, int64_t ldx, const void* w, const void* b, int w_f32,
@@ -1569,24 +1798,35 @@ extern "C" int sd_moe_route(const float* logits, int64_t ld, int32_t* sel_expert
   return SD_OK;
 }
 
-extern "C" int sd_moe_route_rows(const float* x, int64_t ldx, const void* w_router, int w_f32, float* logits,
-                                 int32_t* sel_expert, float* sel_weight, int n_rows, int E, int K, int top,
-                                 int score_kind, int renorm, sd_stream_t stream) {
+extern "C" int sd_moe_route_rows_gated(const float* x, int64_t ldx, const void* w_router, int w_f32, float* logits,
+                                       int32_t* sel_expert, float* sel_weight, int n_rows, int E, int K, int top,
+                                       int score_kind, int renorm, float renorm_eps, float weight_scale,
+                                       const void* w_gate, int n_gate, float* gate_out, sd_stream_t stream) {
   SD_REQUIRE(x && w_router && sel_expert && sel_weight && n_rows >= 1 && E >= 1 && K >= 1 && top >= 1 && top <= E &&
                  ldx >= K,
              SD_ERR_INVALID, "sd_moe_route_rows: bad argument (E=%d top=%d)", E, top);
+  SD_REQUIRE(n_gate >= 0 && (n_gate == 0 || (w_gate && gate_out)), SD_ERR_INVALID,
+             "sd_moe_route_rows: gate rows without their matrix or output");
   SD_REQUIRE(E <= 8192, SD_ERR_UNSUPPORTED, "sd_moe_route_rows: more than 8192 experts");
   hipStream_t st = (hipStream_t)stream;
   const int nthr = 64 * (E >= 16 ? 16 : (E >= 8 ? 8 : 4));   // a wave per expert, up to 16 at a time
   if (w_f32)
-    moe_route_rows_kernel<float><<<n_rows, nthr, sizeof(float) * E, st>>>(x, ldx, (const float*)w_router, logits, sel_expert,
-                                                                          sel_weight, E, K, top, score_kind, renorm, 0);
+    moe_route_rows_kernel<float><<<n_rows, nthr, sizeof(float) * E, st>>>(
+        x, ldx, (const float*)w_router, logits, sel_expert, sel_weight, E, K, top, score_kind, renorm, 0, renorm_eps,
+        weight_scale, (const float*)w_gate, n_gate, gate_out);
   else
-    moe_route_rows_kernel<bf16_t><<<n_rows, nthr, sizeof(float) * E, st>>>(x, ldx, (const bf16_t*)w_router, logits,
-                                                                          sel_expert, sel_weight, E, K, top, score_kind,
-                                                                          renorm, 1);
+    moe_route_rows_kernel<bf16_t><<<n_rows, nthr, sizeof(float) * E, st>>>(
+        x, ldx, (const bf16_t*)w_router, logits, sel_expert, sel_weight, E, K, top, score_kind, renorm, 1, renorm_eps,
+        weight_scale, (const bf16_t*)w_gate, n_gate, gate_out);
   SD_CHECK_LAUNCH("sd_moe_route_rows");
   return SD_OK;
+}
+
+extern "C" int sd_moe_route_rows(const float* x, int64_t ldx, const void* w_router, int w_f32, float* logits,
+                                 int32_t* sel_expert, float* sel_weight, int n_rows, int E, int K, int top,
+                                 int score_kind, int renorm, sd_stream_t stream) {
+  return sd_moe_route_rows_gated(x, ldx, w_router, w_f32, logits, sel_expert, sel_weight, n_rows, E, K, top, score_kind,
+                                 renorm, 0.f, 1.f, nullptr, 0, nullptr, stream);
 }
 
 extern "C" size_t sd_moe_experts_scratch_bytes(int n_rows, int top, int E, int F, int W) {
@@ -1603,7 +1843,7 @@ extern "C" int sd_moe_experts(const float* x, const void* x_bf16, int64_t ldx, c
   SD_REQUIRE(x && sel_expert && sel_weight && w_gate_up && w_down && out && scratch, SD_ERR_INVALID,
              "sd_moe_experts: null argument");
   SD_REQUIRE(n_rows >= 1 && top >= 1 && E >= 1 && F >= 1 && W >= 1 && ldx >= W, SD_ERR_INVALID, "sd_moe_experts: bad shape");
-  SD_REQUIRE(act_kind == 0, SD_ERR_UNSUPPORTED, "sd_moe_experts: activation %d is not provided", act_kind);
+  SD_REQUIRE(act_kind == 0 || act_kind == 1, SD_ERR_UNSUPPORTED, "sd_moe_experts: activation %d is not provided", act_kind);
   const MoeScratch p = moe_plan(n_rows, top, E, F);
   SD_REQUIRE(scratch_bytes >= p.total, SD_ERR_WORKSPACE, "sd_moe_experts: scratch %zu < %zu bytes", scratch_bytes, p.total);
   SD_REQUIRE(sd_aligned16(scratch), SD_ERR_INVALID, "sd_moe_experts: scratch unaligned");
@@ -1634,15 +1874,19 @@ extern "C" int sd_moe_experts(const float* x, const void* x_bf16, int64_t ldx, c
   }
   if (w_f32) {
     moe_gate_up_kernel<float><<<dim3((F + 63) / 64, tiles_y), 256, 0, st>>>(x, ldx, perm, tiles, n_tiles, sel_weight,
-                                                                            (const float*)w_gate_up, act, top, F, W, scale_input, 0);
+                                                                            (const float*)w_gate_up, act, top, F, W, scale_input, 0, act_kind);
     SD_CHECK_LAUNCH("sd_moe_experts (gate, up)");
     moe_down_kernel<float><<<dim3((W + 63) / 64, tiles_y), 256, 0, st>>>(act, perm, tiles, n_tiles, sel_weight,
                                                                          (const float*)w_down, out, W, F, scale_input);
   } else if (!tiles && W % 8 == 0 && F % 8 == 0 && W <= kGemvMaxK && F <= kGemvMaxK && sd_aligned16(w_gate_up) &&
              sd_aligned16(w_down)) {
     bf16_t* act_b = (bf16_t*)act;
-    moe_gemv_gate_up_kernel<<<dim3((F + 7) / 8, n), 256, sizeof(float) * W, st>>>(
-        x, ldx, sel_expert, sel_weight, (const bf16_t*)w_gate_up, act_b, top, F, W, scale_input);
+    if (act_kind == 0)
+      moe_gemv_gate_up_kernel<true><<<dim3((F + 7) / 8, n), 256, sizeof(float) * W, st>>>(
+          x, ldx, sel_expert, sel_weight, (const bf16_t*)w_gate_up, act_b, top, F, W, scale_input);
+    else
+      moe_gemv_gate_up_kernel<false><<<dim3((F + 7) / 8, n), 256, sizeof(float) * W, st>>>(
+          x, ldx, sel_expert, sel_weight, (const bf16_t*)w_gate_up, act_b, top, F, W, scale_input);
     SD_CHECK_LAUNCH("sd_moe_experts (gate, up)");
     moe_gemv_down_kernel<<<dim3((W + 15) / 16, n), 256, sizeof(float) * F, st>>>(
         act_b, sel_expert, sel_weight, (const bf16_t*)w_down, out, W, F, scale_input);
@@ -1651,14 +1895,18 @@ extern "C" int sd_moe_experts(const float* x, const void* x_bf16, int64_t ldx, c
     bf16_t* act_b = (bf16_t*)act;
     const dim3 g1((F + 127) / 128, tiles_y), g2((W + 127) / 128, tiles_y);
     const bf16_t* xb = (const bf16_t*)x_bf16;
-    moe_gate_up_mfma_kernel<2, 512><<<g1, 256, 0, st>>>(x, xb, ldx, perm, tiles, n_tiles, sel_weight,
-                                                        (const bf16_t*)w_gate_up, act_b, top, F, W, scale_input);
+    if (act_kind == 0)
+      moe_gate_up_mfma_kernel<2, 512, true><<<g1, 256, 0, st>>>(x, xb, ldx, perm, tiles, n_tiles, sel_weight,
+                                                                (const bf16_t*)w_gate_up, act_b, top, F, W, scale_input);
+    else
+      moe_gate_up_mfma_kernel<2, 512, false><<<g1, 256, 0, st>>>(x, xb, ldx, perm, tiles, n_tiles, sel_weight,
+                                                                 (const bf16_t*)w_gate_up, act_b, top, F, W, scale_input);
     SD_CHECK_LAUNCH("sd_moe_experts (gate, up)");
     moe_down_mfma_kernel<2, 512><<<g2, 256, 0, st>>>(act_b, perm, tiles, n_tiles, sel_weight, (const bf16_t*)w_down,
                                                      out, W, F, scale_input);
   } else {
     moe_gate_up_kernel<bf16_t><<<dim3((F + 63) / 64, tiles_y), 256, 0, st>>>(x, ldx, perm, tiles, n_tiles, sel_weight,
-                                                                             (const bf16_t*)w_gate_up, act, top, F, W, scale_input, 1);
+                                                                             (const bf16_t*)w_gate_up, act, top, F, W, scale_input, 1, act_kind);
     SD_CHECK_LAUNCH("sd_moe_experts (gate, up)");
     moe_down_kernel<bf16_t><<<dim3((W + 63) / 64, tiles_y), 256, 0, st>>>(act, perm, tiles, n_tiles, sel_weight,
                                                                           (const bf16_t*)w_down, out, W, F, scale_input);
@@ -1676,6 +1924,27 @@ extern "C" int sd_postnorm_residual(float* x, const float* a, int n_a, float sa,
   else
     postnorm_residual_kernel<bf16_t><<<n_rows, 256, 0, st>>>(x, a, n_a, sa, b, sb, (const bf16_t*)w, eps, (bf16_t*)x_bf16, W);
   SD_CHECK_LAUNCH("sd_postnorm_residual");
+  return SD_OK;
+}
+
+extern "C" int sd_residual_norm(float* x, const float* a, int n_a, const float* b, const float* b_gate, int64_t ldg,
+                                const void* w_post, const void* add, const void* w_next, int w_f32, float eps,
+                                float* x_copy, float* h, void* h_bf16, int n_rows, int W, sd_stream_t stream) {
+  SD_REQUIRE(x && n_rows >= 1 && W >= 1 && (!a || (w_post && n_a >= 1)) && (!b || a) && (!b_gate || (b && ldg >= 1)) &&
+                 (!w_next || h || h_bf16),
+             SD_ERR_INVALID, "sd_residual_norm: bad argument");
+  SD_REQUIRE((size_t)W * sizeof(float) <= 60 * 1024, SD_ERR_UNSUPPORTED, "sd_residual_norm: width %d above 15360", W);
+  hipStream_t st = (hipStream_t)stream;
+  const size_t lds = (size_t)W * sizeof(float);
+  if (w_f32)
+    residual_norm_kernel<float><<<n_rows, 256, lds, st>>>(x, a, n_a, b, b_gate, ldg, (const float*)w_post,
+                                                          (const float*)add, (const float*)w_next, eps, x_copy, h,
+                                                          (bf16_t*)h_bf16, W, 0);
+  else
+    residual_norm_kernel<bf16_t><<<n_rows, 256, lds, st>>>(x, a, n_a, b, b_gate, ldg, (const bf16_t*)w_post,
+                                                           (const bf16_t*)add, (const bf16_t*)w_next, eps, x_copy, h,
+                                                           (bf16_t*)h_bf16, W, 1);
+  SD_CHECK_LAUNCH("sd_residual_norm");
   return SD_OK;
 }
 

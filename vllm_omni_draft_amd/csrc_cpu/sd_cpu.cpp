@@ -1540,6 +1540,29 @@ extern "C" int sd_moe_experts(const float*, const void*, int64_t, const int32_t*
 }
 extern "C" int sd_postnorm_residual(float*, const float*, int, float, const float*, float, const void*, int, float,
                                     void*, int, int, sd_stream_t) { UNSUPPORTED("sd_postnorm_residual"); }
+extern "C" size_t sd_masked_softmax_attention_scratch_bytes(int, int, int, int, int, int, int) { return 0; }
+extern "C" int sd_masked_softmax_attention(const float*, int64_t, const void*, const void*, int, const int32_t*,
+                                           const int32_t*, const int32_t*, int, int, int, int, int, int, int, int, int,
+                                           int, float, float, const float*, float*, void*, void*, size_t, sd_stream_t) {
+  UNSUPPORTED("sd_masked_softmax_attention");
+}
+extern "C" int sd_qk_head_norm_append(float*, int, const void*, float*, int, int, const void*, const float*, int,
+                                      int64_t, int, float, void*, void*, const int32_t*, const int32_t*,
+                                      const int32_t*, int, int, int, sd_stream_t) {
+  UNSUPPORTED("sd_qk_head_norm_append");
+}
+extern "C" int sd_head_gate_rows(float*, int64_t, const float*, int64_t, void*, int64_t, int, int, int, int,
+                                 sd_stream_t) { UNSUPPORTED("sd_head_gate_rows"); }
+extern "C" int sd_act_rows(const float*, const float*, int64_t, float*, int64_t, void*, int64_t, int, int, int, int,
+                           sd_stream_t) { UNSUPPORTED("sd_act_rows"); }
+extern "C" int sd_moe_route_rows_gated(const float*, int64_t, const void*, int, float*, int32_t*, float*, int, int, int,
+                                       int, int, int, float, float, const void*, int, float*, sd_stream_t) {
+  UNSUPPORTED("sd_moe_route_rows_gated");
+}
+extern "C" int sd_residual_norm(float*, const float*, int, const float*, const float*, int64_t, const void*, const void*,
+                                const void*, int, float, float*, float*, void*, int, int, sd_stream_t) {
+  UNSUPPORTED("sd_residual_norm");
+}
 extern "C" int sd_scale_rows(float*, int64_t, float, int, int, sd_stream_t) { UNSUPPORTED("sd_scale_rows"); }
 extern "C" sd_seq_model* sd_seq_model_create(const sd_seq_model_desc*) {
   set_error("sd_seq_model_create: not provided by the CPU build of the library");

@@ -148,7 +148,9 @@ class SeqCache:
     means pk / pv f32 [pages, kv_heads, pooled slots per page, dim | vdim]; one page table per
     slot serves all window layers.  Latent attention keeps one row [kv_rank + rot_dim] per token
     in k only; a state-space recurrence keeps state[layer] [slots, heads, state, vdim] and the
-    tail of its convolution's inputs conv[layer] f32 [slots, taps - 1, channels]."""
+    tail of its convolution's inputs conv[layer] f32 [slots, taps - 1, channels].  The tensors are
+    keyed by the layer's place in the order of running (cfg.runs): a layer that runs several
+    times over keeps a cache for every pass."""
 
     def __init__(self, cfg, dtype: torch.dtype, max_seqs: int, num_pages: int, max_seq_len: int,
                  device="cuda"):
@@ -167,8 +169,8 @@ class SeqCache:
         self.pv: Dict[int, torch.Tensor] = {}
         self.conv: Dict[int, torch.Tensor] = {}
         self.has_pages = False
-        for i, l in enumerate(cfg.layers):
-            m = l.mixer
+        for i, (li, _) in enumerate(cfg.runs):
+            m = cfg.layers[li].mixer
             if m.kind == "latent_attention":
                 # one row per token serves as key and value: the latent, then the shared rotated part
                 self.has_pages = True
@@ -181,6 +183,10 @@ class SeqCache:
                 self.state[i] = torch.zeros(max_seqs, sd.heads, sd.state, sd.vdim, dtype=torch.float32, device=device)
                 self.conv[i] = torch.zeros(max_seqs, max(sd.taps - 1, 1), sd.conv_channels, dtype=torch.float32,
                                            device=device)
+            elif m.kind == "softmax_attention":
+                self.has_pages = True
+                self.k[i] = torch.zeros(num_pages, m.kv_heads, PAGE, m.dim, dtype=dtype, device=device)
+                self.v[i] = torch.zeros(num_pages, m.kv_heads, PAGE, m.vdim, dtype=dtype, device=device)
             elif m.kind == "attention":
                 self.has_pages = True
                 ps = ops.pooled_slots_per_page(PAGE, m.pool)

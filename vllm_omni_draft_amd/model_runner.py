@@ -201,7 +201,7 @@ class DecoderModel:
 
 
 # ---------------------------------------------------------------------------------------------
-_MIX_KIND = {"retention": 0, "gla": 1, "attention": 2, "latent_attention": 3, "parallel": 4}
+_MIX_KIND = {"retention": 0, "gla": 1, "attention": 2, "latent_attention": 3, "parallel": 4, "softmax_attention": 5}
 
 
 class SeqModel:
@@ -219,7 +219,7 @@ class SeqModel:
         self.cfg = weights.cfg
         cfg = self.cfg
         f32 = weights.dtype == torch.float32
-        layers = (_lib.SeqLayer * cfg.n_layers)()
+        layers = (_lib.SeqLayer * cfg.n_runs)()
 
         def rm(w):   # a row-major matrix, or nothing
             return None if w is None or isinstance(w, ops.TiledWeight) else w.data_ptr()
@@ -227,8 +227,42 @@ class SeqModel:
         def tl(w):   # a tiled matrix, or nothing
             return w.data.data_ptr() if isinstance(w, ops.TiledWeight) else None
 
-        for i, (spec, t) in enumerate(zip(cfg.layers, weights.layers)):
+        for i, (li, lap) in enumerate(cfg.runs):
+            spec, t = cfg.layers[li], weights.layers[li]
             m = spec.mixer
+            if cfg.block == "sandwich":
+                # one descriptor per run: a repeated layer's weights with the cache of its pass; the
+                # first layer of a pass adds the pass's vector to the stream
+                ex = spec.experts
+                step = None
+                if lap is not None and li == cfg.loop["start"]:
+                    step = weights.loop_step[lap].data_ptr()
+                acts = {"relu": 0, "silu": 1, "relu2": 2}
+                layers[i] = _lib.SeqLayer(
+                    kind=_MIX_KIND[m.kind], block=2, heads=m.heads, kv_heads=m.kv_heads, dim=m.dim, vdim=m.vdim,
+                    ff=spec.ff, rot_dims=m.rot_dims, rot_layout=int(m.rot_layout == "interleaved"),
+                    inv_freq=_ptr(t.inv_freq), rot_mag=t.rot_mag, score_scale=m.scale,
+                    window=m.window or 0x7fffffff, chunk=m.chunk, softcap=m.softcap, sinks=_ptr(t.sinks),
+                    head_gate=int(m.head_gate), qk_head_norm=int(m.qk_head_norm),
+                    norm_w=_ptr(t.norm_w), norm2_w=_ptr(t.norm2_w), post_norm_w=_ptr(t.post_norm_w),
+                    post_norm2_w=_ptr(t.post_norm2_w), pre_add=step, w_in=rm(t.w_in), w_in_tiled=tl(t.w_in),
+                    w_o=rm(t.w_o), w_o_tiled=tl(t.w_o), kv_rank=m.kv_rank, rot_dim=m.rot_dim,
+                    dkv_norm_w=_ptr(t.dkv_norm_w), w_uk_t=_ptr(t.w_uk_t), w_uv=_ptr(t.w_uv),
+                    q_norm_w=_ptr(t.q_norm_w), k_norm_w=_ptr(t.k_norm_w),
+                    k_cache=_ptr(cache.k.get(i)), v_cache=_ptr(cache.v.get(i)),
+                    w_ff_in=rm(t.w_ff_in), w_ff_in_tiled=tl(t.w_ff_in), w_down=rm(t.w_down),
+                    w_down_tiled=tl(t.w_down), ff_act=acts[spec.ff_act],
+                    n_experts=ex.experts if ex else 0, top=ex.top if ex else 0, expert_ff=ex.ff if ex else 0,
+                    w_router=_ptr(t.w_router), w_gate_up=_ptr(t.w_gate_up), w_down_e=_ptr(t.w_down_e),
+                    expert_act=int(ex.act == "relu2") if ex else 0,
+                    route_score=int(ex.score == "softmax") if ex else 0, route_renorm=int(ex.renorm) if ex else 0,
+                    expert_scale_input=int(ex.scale_input) if ex else 0,
+                    route_renorm_eps=ex.renorm_eps if ex else 0.0, route_scale=ex.scale if ex else 1.0,
+                    shared_ff=ex.shared_ff if ex else 0, shared_act=(2 if ex.act == "relu2" else 1) if ex else 0,
+                    w_shared_in=rm(t.w_shared_in), w_shared_in_tiled=tl(t.w_shared_in),
+                    w_shared_down=rm(t.w_shared_down), w_shared_down_tiled=tl(t.w_shared_down),
+                    w_shared_gate=_ptr(t.w_shared_gate))
+                continue
             if cfg.block == "postnorm":
                 sd, ex = m.ssd, spec.experts
                 layers[i] = _lib.SeqLayer(
@@ -266,10 +300,10 @@ class SeqModel:
                 state=_ptr(cache.state.get(i)) if rec else None,
                 k_cache=_ptr(cache.k.get(i)), v_cache=_ptr(cache.v.get(i)),
                 pk_cache=_ptr(cache.pk.get(i)), pv_cache=_ptr(cache.pv.get(i)))
-        desc = _lib.SeqModelDesc(n_layers=cfg.n_layers, width=cfg.width, vocab=cfg.vocab,
+        desc = _lib.SeqModelDesc(n_layers=cfg.n_runs, width=cfg.width, vocab=cfg.vocab,
                                  weights_f32=int(f32), norm_eps=cfg.norm_eps, embed=_ptr(weights.embed),
                                  head_tiled=tl(weights.head_tiled), final_norm_w=_ptr(weights.final_norm_w), layers=layers,
-                                 plain_norm=int(cfg.block == "postnorm"), embed_scale=cfg.embed_scale,
+                                 plain_norm=int(cfg.block != "gated"), embed_scale=cfg.embed_scale,
                                  bigram=_ptr(weights.bigram), buckets=(cfg.bigram or {}).get("buckets", 0),
                                  mul_prev=(cfg.bigram or {}).get("mul_prev", 0),
                                  mul_cur=(cfg.bigram or {}).get("mul_cur", 0), head=_ptr(weights.head),
@@ -319,8 +353,8 @@ class SeqModel:
                       or logits.numel() < n_out * self.cfg.vocab):
             raise _lib.SdError("wanted rows need int32 out_rows and contiguous float32 logits [n_out, vocab]")
         if layer_out is not None and (layer_out.dtype != torch.float32 or not layer_out.is_contiguous()
-                                      or layer_out.numel() < self.cfg.n_layers * n_rows * self.cfg.width):
-            raise _lib.SdError("layer_out must be contiguous float32 [n_layers, n_rows, width]")
+                                      or layer_out.numel() < self.cfg.n_runs * n_rows * self.cfg.width):
+            raise _lib.SdError("layer_out must be contiguous float32 [layer runs, n_rows, width]")
         self._ensure_workspace(n_rows, n_out)
         c = self.cache
         batch = _lib.SeqBatch(n_rows=n_rows, n_entries=n_entries, tokens=tokens.data_ptr(),

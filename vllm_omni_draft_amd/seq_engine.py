@@ -95,7 +95,8 @@ class SeqEngine:
         """entries: (request id, its next tokens, indices among them whose logits are wanted).
         A request is admitted at its first entry.  Returns the wanted logits, f32 [n, vocab] on
         the device, in the order of the entries and of their indices (and, with layer_out, the
-        residual after every layer, [n_layers, rows, width])."""
+        residual after every layer run, [layer runs, rows, width]; a layer that runs several times
+        over counts each time)."""
         plan = []
         seen = set()
         for rid, toks, want in entries:
@@ -119,7 +120,7 @@ class SeqEngine:
         total = sum(len(t) for _, t, _ in plan)
         if layer_out and total > self.cfg.max_rows:
             raise ValueError("layer_out needs a step of at most max_rows rows")
-        trace = (torch.empty(self.model_cfg.n_layers, total, self.model_cfg.width, dtype=torch.float32,
+        trace = (torch.empty(self.model_cfg.n_runs, total, self.model_cfg.width, dtype=torch.float32,
                              device=self.device) if layer_out else None)
         # cut the step into passes of at most max_rows rows (an entry may span passes)
         done = [0] * len(plan)

@@ -352,8 +352,16 @@ class SeqLayerTensors:
     s_norm_w: Optional[torch.Tensor] = None
     w_o2: object = None
     w_router: Optional[torch.Tensor] = None    # routed experts
-    w_gate_up: Optional[torch.Tensor] = None   # [experts, 2*ff, width]
+    w_gate_up: Optional[torch.Tensor] = None   # [experts, 2*ff, width] ([experts, ff, width]: experts of two matrices)
     w_down_e: Optional[torch.Tensor] = None    # [experts, width, ff]
+    # layers normed before and after their sublayers (norm_w / norm2_w before, these after)
+    post_norm_w: Optional[torch.Tensor] = None
+    post_norm2_w: Optional[torch.Tensor] = None
+    sinks: Optional[torch.Tensor] = None       # f32 [heads]
+    w_ff_in: object = None                     # [2*ff, width]: gate rows, then up rows
+    w_shared_in: object = None                 # a shared expert: [shared_ff, width]
+    w_shared_down: object = None               # [width, shared_ff]
+    w_shared_gate: Optional[torch.Tensor] = None   # [1, width]
 
 
 @dataclass
@@ -366,13 +374,14 @@ class SeqModelWeights:
     head_tiled: Optional["ops.TiledWeight"] = None   # the head's matrix once more, tiled
     head: Optional[torch.Tensor] = None              # an untied head, row-major
     bigram: Optional[torch.Tensor] = None            # [buckets + 1, width]
+    loop_step: Optional[torch.Tensor] = None         # [times, width]: added to the stream before each pass
 
     def tensors(self):
         yield self.embed
         yield self.final_norm_w
         if self.head_tiled is not None:
             yield self.head_tiled.data
-        for t in (self.head, self.bigram):
+        for t in (self.head, self.bigram, self.loop_step):
             if t is not None:
                 yield t
         for l in self.layers:
@@ -413,6 +422,12 @@ def seq_from_state_dict(cfg, state: Dict[str, torch.Tensor], device="cuda",
             return ops.tile_weights(d, ops.TILE_PLAIN)
         return d
 
+    if cfg.block == "sandwich":
+        layers = [_sandwich_layer(cfg, i, get, dev, mat) for i in range(cfg.n_layers)]
+        head = mat(get("head", (cfg.vocab, W)))
+        return SeqModelWeights(cfg, dtype, dev(get("embed", (cfg.vocab, W))), dev(get("final.norm", (W,))), layers,
+                               head if isinstance(head, ops.TiledWeight) else None, dev(get("head", (cfg.vocab, W))),
+                               loop_step=dev(get("loop.step", (cfg.loop["times"], W))) if cfg.loop else None)
     if cfg.block == "postnorm":
         layers = [_postnorm_layer(cfg, i, get, dev, mat) for i in range(cfg.n_layers)]
         head_t = get("embed" if cfg.tied_head else "head", (cfg.vocab, W))
@@ -501,6 +516,58 @@ def _postnorm_layer(cfg, i: int, get, dev, mat) -> SeqLayerTensors:
     return lt
 
 
+def _sandwich_layer(cfg, i: int, get, dev, mat) -> SeqLayerTensors:
+    """Layer i of a model whose layers are normed before and after their sublayers: the matrices
+    that read the mixer's normed input stacked into w_in (the head gates last), per-head key
+    expansions transposed, a gated feed-forward's two input matrices stacked, the experts'
+    matrices stacked per layer."""
+    l, p, W = cfg.layers[i], f"l{i}.", cfg.width
+    m = l.mixer
+    H, G, dk, dv = m.heads, m.kv_heads, m.dim, m.vdim
+    if m.kind == "latent_attention":
+        rk, dr = m.kv_rank, m.rot_dim
+        parts = [get(p + "mix.q", (H * (dk + dr), W)), get(p + "mix.dkv", (rk + dr, W))]
+        if m.head_gate:
+            parts.append(get(p + "mix.g", (H, W)))
+        lt = SeqLayerTensors(norm_w=dev(get(p + "norm1", (W,))), w_in=mat(torch.cat([t.float() for t in parts])),
+                             w_o=mat(get(p + "mix.o", (W, H * dv))), r1_bias=None)
+        lt.dkv_norm_w = dev(get(p + "mix.dkv.norm", (rk,)))
+        lt.w_uk_t = dev(get(p + "mix.uk", (H * dk, rk)).view(H, dk, rk).transpose(1, 2))
+        lt.w_uv = dev(get(p + "mix.uv", (H * dv, rk)))
+        if m.sink:
+            lt.sinks = dev(get(p + "mix.sink", (H,)), torch.float32)
+        if m.rot_dims:
+            i2 = torch.arange(m.rot_dims // 2, dtype=torch.float64)
+            lt.inv_freq = dev(torch.tensor(m.rot_base, dtype=torch.float64) ** (-2.0 * i2 / m.rot_dims), torch.float64)
+    else:
+        parts = [get(p + "mix.q", (H * dk, W)), get(p + "mix.k", (G * dk, W)), get(p + "mix.v", (G * dv, W))]
+        lt = SeqLayerTensors(norm_w=dev(get(p + "norm1", (W,))), w_in=mat(torch.cat([t.float() for t in parts])),
+                             w_o=mat(get(p + "mix.o", (W, H * dv))), r1_bias=None)
+        lt.q_norm_w, lt.k_norm_w = dev(get(p + "mix.q.norm", (dk,))), dev(get(p + "mix.k.norm", (dk,)))
+    lt.post_norm_w = dev(get(p + "norm1b", (W,)))
+    ex = l.experts
+    if l.ff or ex is not None:
+        lt.norm2_w, lt.post_norm2_w = dev(get(p + "norm2", (W,))), dev(get(p + "norm2b", (W,)))
+    if l.ff:
+        lt.w_ff_in = mat(torch.cat([get(p + "mlp.gate", (l.ff, W)).float(), get(p + "mlp.up", (l.ff, W)).float()]))
+        lt.w_down = mat(get(p + "mlp.down", (W, l.ff)))
+    if ex is not None:
+        gated = ex.act == "silu"
+        lt.w_router = dev(get(p + "mlp.router", (ex.experts, W)))
+        lt.w_gate_up = dev(torch.stack([
+            torch.cat([get(p + f"mlp.e{e}.gate", (ex.ff, W)), get(p + f"mlp.e{e}.up", (ex.ff, W))]) if gated
+            else get(p + f"mlp.e{e}.up", (ex.ff, W)) for e in range(ex.experts)]))
+        lt.w_down_e = dev(torch.stack([get(p + f"mlp.e{e}.down", (W, ex.ff)) for e in range(ex.experts)]))
+        if ex.shared_ff:
+            F = ex.shared_ff
+            lt.w_shared_in = mat(torch.cat([get(p + "mlp.shared.gate", (F, W)).float(), get(p + "mlp.shared.up", (F, W)).float()])
+                                 if gated else get(p + "mlp.shared.up", (F, W)))
+            lt.w_shared_down = mat(get(p + "mlp.shared.down", (W, F)))
+            if ex.shared_gate:
+                lt.w_shared_gate = dev(get(p + "mlp.shared.sg", (1, W)))
+    return lt
+
+
 def seq_from_safetensors_dir(cfg, model_dir: str, device="cuda",
                              dtype: torch.dtype = torch.bfloat16) -> SeqModelWeights:
     from safetensors import safe_open
@@ -527,6 +594,8 @@ def seq_random_state(cfg, seed: int = 0) -> Dict[str, torch.Tensor]:
 
     if cfg.block == "postnorm":
         return _postnorm_random_state(cfg, rn)
+    if cfg.block == "sandwich":
+        return _sandwich_random_state(cfg, rn)
     st = {"embed": rn(cfg.vocab, W, s=1.0), "final.norm": rn(W, s=0.1)}
     for i, l in enumerate(cfg.layers):
         m, p = l.mixer, f"l{i}."
@@ -585,6 +654,47 @@ def _postnorm_random_state(cfg, rn) -> Dict[str, torch.Tensor]:
             for e in range(ex.experts):
                 st[p + f"mlp.e{e}.gate"], st[p + f"mlp.e{e}.up"] = rn(ex.ff, W, s=W ** -0.5), rn(ex.ff, W, s=W ** -0.5)
                 st[p + f"mlp.e{e}.down"] = rn(W, ex.ff, s=ex.ff ** -0.5)
+    return st
+
+
+def _sandwich_random_state(cfg, rn) -> Dict[str, torch.Tensor]:
+    W = cfg.width
+    st = {"embed": rn(cfg.vocab, W, s=1.0), "final.norm": 1 + rn(W, s=0.1), "head": rn(cfg.vocab, W, s=W ** -0.5)}
+    if cfg.loop:
+        st["loop.step"] = rn(cfg.loop["times"], W, s=0.5)
+    for i, l in enumerate(cfg.layers):
+        m, p = l.mixer, f"l{i}."
+        H, G, dk, dv = m.heads, m.kv_heads, m.dim, m.vdim
+        for nm in ("norm1", "norm1b") + (("norm2", "norm2b") if (l.ff or l.experts) else ()):
+            st[p + nm] = 1 + rn(W, s=0.1)
+        if m.kind == "latent_attention":
+            rk, dr = m.kv_rank, m.rot_dim
+            st[p + "mix.q"] = rn(H * (dk + dr), W, s=W ** -0.5)
+            st[p + "mix.dkv"], st[p + "mix.dkv.norm"] = rn(rk + dr, W, s=W ** -0.5), 1 + rn(rk, s=0.1)
+            st[p + "mix.uk"], st[p + "mix.uv"] = rn(H * dk, rk, s=rk ** -0.5), rn(H * dv, rk, s=rk ** -0.5)
+            if m.sink:
+                st[p + "mix.sink"] = rn(H, s=1.0)
+            if m.head_gate:
+                st[p + "mix.g"] = rn(H, W, s=W ** -0.5)
+        else:
+            st[p + "mix.q"], st[p + "mix.k"] = rn(H * dk, W, s=W ** -0.5), rn(G * dk, W, s=W ** -0.5)
+            st[p + "mix.v"] = rn(G * dv, W, s=W ** -0.5)
+            st[p + "mix.q.norm"], st[p + "mix.k.norm"] = 1 + rn(dk, s=0.1), 1 + rn(dk, s=0.1)
+        st[p + "mix.o"] = rn(W, H * dv, s=(H * dv) ** -0.5)
+        if l.ff:
+            st[p + "mlp.gate"], st[p + "mlp.up"] = rn(l.ff, W, s=W ** -0.5), rn(l.ff, W, s=W ** -0.5)
+            st[p + "mlp.down"] = rn(W, l.ff, s=l.ff ** -0.5)
+        ex = l.experts
+        if ex is not None:
+            st[p + "mlp.router"] = rn(ex.experts, W, s=W ** -0.5)
+            names = [f"e{e}" for e in range(ex.experts)] + (["shared"] if ex.shared_ff else [])
+            for nm in names:
+                F = ex.shared_ff if nm == "shared" else ex.ff
+                if ex.act == "silu":
+                    st[p + f"mlp.{nm}.gate"] = rn(F, W, s=W ** -0.5)
+                st[p + f"mlp.{nm}.up"], st[p + f"mlp.{nm}.down"] = rn(F, W, s=W ** -0.5), rn(W, F, s=F ** -0.5)
+            if ex.shared_ff and ex.shared_gate:
+                st[p + "mlp.shared.sg"] = rn(1, W, s=W ** -0.5)
     return st
 
 
