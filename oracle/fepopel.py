@@ -35,6 +35,34 @@ def rotate_pairs(v, pos, dims, base):
     return v
 
 
+def visible(i, j, chunk=0):
+    """Whether the query at position i sees the key at position j."""
+    return j <= i and (chunk <= 0 or i // chunk == j // chunk)
+
+
+def attend(q, k, v, pos_q, scale, chunk=0, softcap=0.0, sink=None):
+    """q [n, H, dk] at positions pos_q against keys k [T, G, dk] / values v [T, G, dv] at positions
+    0..T-1 -> [n, H, dv].  Head h reads key head h // (H/G).  sink [H]: one more term exp(sink) in
+    the denominator."""
+    n, H, _ = q.shape
+    T, G, _ = k.shape
+    rep = H // G
+    k, v = k.to(F64).repeat_interleave(rep, 1), v.to(F64).repeat_interleave(rep, 1)
+    s = torch.einsum("ihd,jhd->hij", q.to(F64), k) * scale
+    if softcap > 0:
+        s = softcap * torch.tanh(s / softcap)
+    seen = torch.tensor([[visible(int(i), j, chunk) for j in range(T)] for i in pos_q])
+    s = s.masked_fill(~seen[None], -math.inf)
+    mx = s.max(-1).values
+    if sink is not None:
+        mx = torch.maximum(mx, sink.to(F64)[:, None])
+    e = torch.exp(s - mx[..., None])
+    den = e.sum(-1)
+    if sink is not None:
+        den = den + torch.exp(sink.to(F64)[:, None] - mx)
+    return torch.einsum("hij,jhd->ihd", e / den[..., None], v)
+
+
 def latent_attention(h, m, t, pos):
     """h [T, W] -> [T, W].  m: the mixer's sizes and constants; t: its tensors by short name."""
     T = h.shape[0]
@@ -42,22 +70,14 @@ def latent_attention(h, m, t, pos):
     h = h.to(F64)
     q = (h @ t["q"].to(F64).T).view(T, H, dk + dr)
     low = h @ t["dkv"].to(F64).T
-    c = rms_norm(low[:, :rk], t["dkv.norm"], m["eps"])                       # the latent
-    k_rot = rotate_pairs(low[:, rk:], pos, m["rot"]["dims"], m["rot"]["base"])      # [T, dr], shared
+    c = rms_norm(low[:, :rk], t["dkv.norm"], m["eps"])                              # the latent
+    k_rot = rotate_pairs(low[:, rk:], pos, m["rot"]["dims"], m["rot"]["base"])      # [T, dr], shared by the heads
     q_rot = rotate_pairs(q[..., dk:], pos, m["rot"]["dims"], m["rot"]["base"])
-    k = (c @ t["uk"].to(F64).T).view(T, H, dk)
+    k = torch.cat([(c @ t["uk"].to(F64).T).view(T, H, dk), k_rot[:, None, :].expand(T, H, dr)], -1)
     v = (c @ t["uv"].to(F64).T).view(T, H, dv)
-    s = (torch.einsum("ihd,jhd->hij", q[..., :dk], k) + torch.einsum("ihd,jd->hij", q_rot, k_rot)) * m["scale"]
-    causal = pos[:, None] >= pos[None, :]
-    s = s.masked_fill(~causal[None], -math.inf)
-    sink = t["sink"].to(F64)                                                    # [H]
-    mx = torch.maximum(s.max(-1).values, sink[:, None])
-    e = torch.exp(s - mx[..., None])
-    p = e / (e.sum(-1) + torch.exp(sink[:, None] - mx))[..., None]
-    o = torch.einsum("hij,jhd->ihd", p, v)
-    gate = torch.sigmoid(h @ t["g"].to(F64).T)                                  # [T, H]
-    o = o * gate[..., None]
-    return o.reshape(T, H * dv) @ t["o"].to(F64).T
+    o = attend(torch.cat([q[..., :dk], q_rot], -1), k, v, pos, m["scale"], sink=t["sink"])
+    gate = torch.sigmoid(h @ t["g"].to(F64).T)                                      # [T, H]
+    return (o * gate[..., None]).reshape(T, H * dv) @ t["o"].to(F64).T
 
 
 def chunk_attention(h, m, t, pos):
@@ -67,15 +87,8 @@ def chunk_attention(h, m, t, pos):
     q = rms_norm((h @ t["q"].to(F64).T).view(T, H, dk), t["q.norm"], m["eps"])
     k = rms_norm((h @ t["k"].to(F64).T).view(T, G, dk), t["k.norm"], m["eps"])
     v = (h @ t["v"].to(F64).T).view(T, G, dv)
-    rep = H // G
-    k, v = k.repeat_interleave(rep, 1), v.repeat_interleave(rep, 1)
-    s = torch.einsum("ihd,jhd->hij", q, k) * m["scale"]
-    cap = m["softcap"]
-    s = cap * torch.tanh(s / cap)
-    size = m["mask"]["size"]
-    seen = (pos[:, None] >= pos[None, :]) & ((pos[:, None] // size) == (pos[None, :] // size))
-    p = torch.softmax(s.masked_fill(~seen[None], -math.inf), -1)
-    return torch.einsum("hij,jhd->ihd", p, v).reshape(T, H * dv) @ t["o"].to(F64).T
+    o = attend(q, k, v, pos, m["scale"], chunk=m["mask"]["size"], softcap=m["softcap"])
+    return o.reshape(T, H * dv) @ t["o"].to(F64).T
 
 
 def dense_ff(h, t):
@@ -149,3 +162,49 @@ def forward(cfg, state, tokens, layer_out=None):
         if layer_out is not None:
             layer_out.append(x.clone())
     return rms_norm(x, state["final.norm"], eps) @ state["head"].to(F64).T
+
+
+def random_tensors(cfg, seed=0):
+    """Seeded random tensors (bfloat16 values, as float32) under the checkpoint's names."""
+    g = torch.Generator().manual_seed(seed)
+
+    def rn(*shape, s=1.0):
+        return (torch.randn(*shape, generator=g) * s).to(torch.bfloat16).float()
+
+    W, st = cfg["width"], {}
+    st["embed"], st["head"], st["final.norm"] = rn(cfg["vocab"], W), rn(cfg["vocab"], W, s=W ** -0.5), 1 + rn(W, s=0.1)
+    if cfg.get("loop"):
+        st["loop.step"] = rn(cfg["loop"]["times"], W, s=0.5)
+    for i, l in enumerate(cfg["layers"]):
+        m, p = l["mixer"], f"l{i}."
+        H, dk, dv = m["heads"], m["dim"], m["vdim"]
+        st[p + "norm1"], st[p + "norm1b"] = 1 + rn(W, s=0.1), 1 + rn(W, s=0.1)
+        if l["type"] == "latent_attention":
+            rk, dr = m["kv_rank"], m["rot_dim"]
+            st[p + "mix.q"], st[p + "mix.dkv"] = rn(H * (dk + dr), W, s=W ** -0.5), rn(rk + dr, W, s=W ** -0.5)
+            st[p + "mix.dkv.norm"] = 1 + rn(rk, s=0.1)
+            st[p + "mix.uk"], st[p + "mix.uv"] = rn(H * dk, rk, s=rk ** -0.5), rn(H * dv, rk, s=rk ** -0.5)
+            st[p + "mix.sink"], st[p + "mix.g"] = rn(H), rn(H, W, s=W ** -0.5)
+        else:
+            G = m["kv_heads"]
+            st[p + "mix.q"], st[p + "mix.k"] = rn(H * dk, W, s=W ** -0.5), rn(G * dk, W, s=W ** -0.5)
+            st[p + "mix.v"] = rn(G * dv, W, s=W ** -0.5)
+            st[p + "mix.q.norm"], st[p + "mix.k.norm"] = 1 + rn(dk, s=0.1), 1 + rn(dk, s=0.1)
+        st[p + "mix.o"] = rn(W, H * dv, s=(H * dv) ** -0.5)
+        mlp = l.get("mlp")
+        if not mlp:
+            continue
+        st[p + "norm2"], st[p + "norm2b"] = 1 + rn(W, s=0.1), 1 + rn(W, s=0.1)
+        if mlp["kind"] == "dense":
+            F = mlp["ff"]
+            st[p + "mlp.gate"], st[p + "mlp.up"], st[p + "mlp.down"] = rn(F, W, s=W ** -0.5), rn(F, W, s=W ** -0.5), rn(W, F, s=F ** -0.5)
+            continue
+        E, F = mlp["router"]["experts"], mlp["expert"]["ff"]
+        st[p + "mlp.router"] = rn(E, W, s=2 * W ** -0.5)
+        for e in range(E):
+            st[p + f"mlp.e{e}.up"], st[p + f"mlp.e{e}.down"] = rn(F, W, s=W ** -0.5), rn(W, F, s=F ** -0.5)
+        if mlp.get("shared"):
+            Fs = mlp["shared"]["ff"]
+            st[p + "mlp.shared.up"], st[p + "mlp.shared.down"] = rn(Fs, W, s=W ** -0.5), rn(W, Fs, s=Fs ** -0.5)
+            st[p + "mlp.shared.sg"] = rn(1, W, s=W ** -0.5)
+    return st

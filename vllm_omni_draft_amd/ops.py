@@ -1247,6 +1247,119 @@ def window_softmax_attention(q, k_cache, v_cache, row_pos, row_slot, block_table
     return out
 
 
+def masked_softmax_attention(q, k_cache, v_cache, row_pos, row_slot, block_tables, H, G, dk, dv, scale, window=0,
+                             keep_first=0, chunk=0, softcap=0.0, sinks=None, split=True) -> torch.Tensor:
+    """window_softmax_attention with the further masks of sd_masked_softmax_attention: window 0
+    sees every earlier token, chunk > 0 only the keys of the row's own chunk; softcap > 0 caps the
+    scores; sinks f32 [H]: a term without key or value in every head's denominator."""
+    _f32(q, "q")
+    if sinks is not None:
+        _f32(sinks, "sinks")
+    window = int(window) or 0x7fffffff
+    out = torch.empty(q.shape[0], H * dv, dtype=torch.float32, device=q.device)
+    lib = _lib.load()
+    n = int(lib.sd_masked_softmax_attention_scratch_bytes(q.shape[0], H, dv, window, int(keep_first), int(chunk),
+                                                          block_tables.shape[1] * PAGE)) if split else 0
+    scratch = torch.empty(n, dtype=torch.uint8, device=q.device) if n else None
+    _lib.check(lib.sd_masked_softmax_attention(
+        _p(q), q.shape[1], _p(k_cache), _p(v_cache), int(k_cache.dtype == torch.float32), _p(row_pos),
+        _p(row_slot), _p(block_tables), block_tables.shape[1], PAGE, q.shape[0], H, G, dk, dv, window,
+        int(keep_first), int(chunk), float(scale), float(softcap), _p(sinks), _p(out), None, _p(scratch), n,
+        _stream()), "sd_masked_softmax_attention")
+    return out
+
+
+def qk_head_norm_append(q, q_norm_w, k, k_norm_w, v, H, G, dk, dv, eps, k_cache, v_cache, row_pos, row_slot,
+                        block_tables) -> None:
+    """In place on q f32 [rows, H*dk] and k f32 [rows, G*dk] (every head normed by itself, one
+    weight [dk] for the query heads and one for the key heads); appends k and v f32 [rows, G*dv] to
+    the caches.  See sd_qk_head_norm_append."""
+    for t, nm in ((q, "q"), (k, "k"), (v, "v")):
+        _f32(t, nm)
+    buf = torch.cat([q, k, v], dim=1).contiguous()
+    nq, nk = q.shape[1], k.shape[1]
+    _lib.check(_lib.load().sd_qk_head_norm_append(buf.data_ptr(), H, _p(q_norm_w), buf.data_ptr() + 4 * nq, G, dk,
+                                                  _p(k_norm_w), buf.data_ptr() + 4 * (nq + nk), dv, buf.shape[1],
+                                                  _wkind(q_norm_w, "q_norm_w"), float(eps), _p(k_cache), _p(v_cache),
+                                                  _p(row_pos), _p(row_slot), _p(block_tables), block_tables.shape[1],
+                                                  PAGE, q.shape[0], _stream()), "sd_qk_head_norm_append")
+    q.copy_(buf[:, :nq])
+    k.copy_(buf[:, nq:nq + nk])
+
+
+def latent_kv_prep(kv, kv_norm_w, kv_rank, rot_dim, eps, rot_dims, inv_freq, k_cache, row_pos, row_slot,
+                   block_tables, mag=1.0, layout=1) -> None:
+    """latent_prep for queries that have no latent: in place on kv f32 [rows, kv_rank + rot_dim],
+    which is appended to k_cache."""
+    _f32(kv, "kv")
+    _lib.check(_lib.load().sd_latent_prep(None, 0, None, None, 0, _p(kv), kv_rank, rot_dim, _p(kv_norm_w), kv.shape[1],
+                                          _wkind(kv_norm_w, "kv_norm_w"), float(eps), rot_dims, layout, _p(inv_freq),
+                                          float(mag), _p(k_cache), _p(row_pos), _p(row_slot), _p(block_tables),
+                                          block_tables.shape[1], PAGE, kv.shape[0], _stream()), "sd_latent_prep")
+
+
+def head_gate_rows(y, z, H, dv) -> None:
+    """y f32 [rows, H*dv] *= sigmoid(z f32 [rows, H]) per (row, head), in place."""
+    _f32(y, "y")
+    _f32(z, "z")
+    _lib.check(_lib.load().sd_head_gate_rows(_p(y), y.shape[1], _p(z), z.shape[1], None, 0, y.shape[0], H, dv, 0,
+                                             _stream()), "sd_head_gate_rows")
+
+
+ACT_KINDS = {"relu": 0, "silu": 1, "relu2": 2}
+
+
+def act_rows(gate, up, kind: str, bf16_copy: bool = False):
+    """A feed-forward's activation over f32 [rows, F]: "relu" / "silu": act(gate) * up; "relu2":
+    relu(gate)^2 (up None).  Returns f32 [rows, F] (and its bfloat16 copy)."""
+    _f32(gate, "gate")
+    n, F = gate.shape
+    buf = torch.cat([gate, up], dim=1).contiguous() if up is not None else gate.contiguous()
+    out = torch.empty(n, F, dtype=torch.float32, device=gate.device)
+    ob = torch.empty(n, F, dtype=torch.bfloat16, device=gate.device) if bf16_copy else None
+    _lib.check(_lib.load().sd_act_rows(buf.data_ptr(), buf.data_ptr() + 4 * F if up is not None else None,
+                                       buf.shape[1], _p(out), F, _p(ob), F, n, F, ACT_KINDS[kind], int(bf16_copy),
+                                       _stream()), "sd_act_rows")
+    return (out, ob) if bf16_copy else out
+
+
+def moe_route_rows_gated(x, w_router, top, score="softmax", renorm=True, renorm_eps=0.0, weight_scale=1.0,
+                         w_gate=None):
+    """moe_route_rows with weights = chosen / (sum + renorm_eps) * weight_scale, and the products
+    of x with the rows of w_gate [n_gate, K]: (experts, weights, logits, gates f32 [rows, n_gate]
+    or None)."""
+    _f32(x, "x")
+    n, K = x.shape
+    E = w_router.shape[0]
+    sel_e = torch.empty(n, top, dtype=torch.int32, device=x.device)
+    sel_w = torch.empty(n, top, dtype=torch.float32, device=x.device)
+    logits = torch.empty(n, E, dtype=torch.float32, device=x.device)
+    ng = w_gate.shape[0] if w_gate is not None else 0
+    gates = torch.empty(n, ng, dtype=torch.float32, device=x.device) if ng else None
+    _lib.check(_lib.load().sd_moe_route_rows_gated(
+        _p(x), K, _p(w_router), _wkind(w_router, "w_router"), _p(logits), _p(sel_e), _p(sel_w), n, E, K, top,
+        {"sigmoid": 0, "softmax": 1}[score], int(renorm), float(renorm_eps), float(weight_scale), _p(w_gate), ng,
+        _p(gates), _stream()), "sd_moe_route_rows_gated")
+    return sel_e, sel_w, logits, gates
+
+
+def residual_norm(x, a=None, w_post=None, n_a=1, b=None, b_gate=None, add=None, w_next=None, eps=1e-5,
+                  want_copy=False):
+    """sd_residual_norm, in place on x f32 [rows, W]: x += rms_norm(sum of each row's n_a rows of a
+    (+ sigmoid(b_gate) * b)) * w_post; then x += add; returns (the rows before `add` if want_copy,
+    rms_norm(x) * w_next if w_next is given)."""
+    _f32(x, "x")
+    n, W = x.shape
+    ref = w_post if w_post is not None else (w_next if w_next is not None else add)
+    copy = torch.empty_like(x) if want_copy else None
+    h = torch.empty_like(x) if w_next is not None else None
+    _lib.check(_lib.load().sd_residual_norm(_p(x), _p(a), int(n_a), _p(b), _p(b_gate),
+                                            b_gate.shape[1] if b_gate is not None else 0, _p(w_post), _p(add),
+                                            _p(w_next), _wkind(ref, "w"), float(eps), _p(copy), _p(h), None, n, W,
+                                            _stream()), "sd_residual_norm")
+    return copy, h
+
+
 def matmul_rows_batched(x, w) -> torch.Tensor:
     """x f32 [M, B, K], w [B, N, K] -> f32 [M, B, N]: product b uses w[b]."""
     _f32(x, "x")
@@ -1320,9 +1433,9 @@ def moe_route_rows(x, w_router, top, score="sigmoid", renorm=False):
     return sel_e, sel_w, logits
 
 
-def moe_experts(x, sel_e, sel_w, w_gate_up, w_down, scale_input=True) -> torch.Tensor:
+def moe_experts(x, sel_e, sel_w, w_gate_up, w_down, scale_input=True, act="silu") -> torch.Tensor:
     """x f32 [rows, W]; w_gate_up [E, 2F, W], w_down [E, W, F]; returns f32 [rows, top, W]: every
-    chosen expert's result."""
+    chosen expert's result.  act "relu2": experts of two matrices, w_gate_up is [E, F, W]."""
     _f32(x, "x")
     n, W = x.shape
     top, E, F = sel_e.shape[1], w_gate_up.shape[0], w_down.shape[2]
@@ -1331,7 +1444,8 @@ def moe_experts(x, sel_e, sel_w, w_gate_up, w_down, scale_input=True) -> torch.T
     scratch = torch.empty(nb, dtype=torch.uint8, device=x.device)
     out = torch.empty(n, top, W, dtype=torch.float32, device=x.device)
     _lib.check(lib.sd_moe_experts(_p(x), None, W, _p(sel_e), _p(sel_w), _p(w_gate_up), _p(w_down), _wkind(w_down, "w_down"),
-                                  _p(out), n, top, E, F, W, int(scale_input), 0, _p(scratch), nb, _stream()),
+                                  _p(out), n, top, E, F, W, int(scale_input), {"silu": 0, "relu2": 1}[act], _p(scratch),
+                                  nb, _stream()),
                "sd_moe_experts")
     return out
 
