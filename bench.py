@@ -102,14 +102,17 @@ def parse():
     ap.add_argument("--tp-draft", choices=["replicated", "sharded"], default="replicated",
                     help="the draft whole on every rank (no exchange in its passes), or sharded "
                          "like the target with a vocabulary-parallel head")
-    ap.add_argument("--family", choices=["spec", "puguzen", "naburax"], default="spec",
+    ap.add_argument("--family", choices=["spec", "puguzen", "naburax", "fepopel"], default="spec",
                     help="spec: the headline speculative-decoding workload (default).  puguzen: prefill and "
                          "decode throughput of the Puguzen decoder family (recurrent and windowed layers) at "
                          "layer sizes of real models, beside a Llama-style decoder of equal size, with the "
                          "time and memory traffic of its own kernels.  naburax: the same for the Naburax "
                          "family (latent attention, attention beside a state-space recurrence, routed "
-                         "experts), beside the Puguzen family at equal size")
-    ap.add_argument("--seq-sizes", default="w1024,w2048,w4096", help="--family puguzen / naburax: sizes to run")
+                         "experts), beside the Puguzen family at equal size.  fepopel: the same for the "
+                         "Fepopel family (latent attention with a sink over every earlier token, chunked "
+                         "softmax attention, experts of two matrices beside a shared one, a repeated span of "
+                         "layers), beside the Naburax family at equal size")
+    ap.add_argument("--seq-sizes", default="w1024,w2048,w4096", help="--family puguzen / naburax / fepopel: sizes to run")
     return ap.parse_args()
 
 
@@ -957,9 +960,137 @@ def main_nab_family(args):
     print(json.dumps({"metric": "naburax_family_throughput", "unit": "tokens/s", "dtype": "bf16",
                       "data": "synthetic", "n_gpus": 1, "steps": steps, "warmup": warm, "sizes": results}))
 
+# ---------------------------------------------------------------------------------------------
+# --family fepopel
+FEP_SIZES = {
+    "w1024": dict(width=1024, heads=8, kv_heads=2, ff=4096, experts=8, top=2, eff=1024, shared=1024),
+    "w2048": dict(width=2048, heads=16, kv_heads=4, ff=8192, experts=16, top=2, eff=2048, shared=2048),
+    "w4096": dict(width=4096, heads=32, kv_heads=8, ff=14336, experts=16, top=2, eff=4096, shared=4096),
+}
+FEP_CHUNK, FEP_CAP, FEP_LOOP = 1024, 30.0, {"start": 1, "stop": 3, "times": 2}
+
+
+def _fep_config(sz):
+    from vllm_omni_draft_amd.config import ExpertsSpec, MixerSpec, SeqLayerSpec, SeqModelConfig
+    H, G, D = sz["heads"], sz["kv_heads"], SEQ_HEAD
+    lat = MixerSpec("latent_attention", H, D, D, q_rank=0, kv_rank=NAB_KV_RANK, rot_dim=NAB_ROT, rot_dims=NAB_ROT,
+                    rot_base=1e6, rot_layout="interleaved", scale=(D + NAB_ROT) ** -0.5, window=0, sink=True,
+                    head_gate=True)
+    att = MixerSpec("softmax_attention", H, D, D, kv_heads=G, scale=D ** -0.5, window=0, chunk=FEP_CHUNK,
+                    softcap=FEP_CAP, qk_head_norm=True)
+    ex = ExpertsSpec(sz["experts"], sz["top"], sz["eff"], score="softmax", renorm=True, scale_input=False, act="relu2",
+                     renorm_eps=1e-20, scale=1.5, shared_ff=sz["shared"])
+    layers = [SeqLayerSpec(lat, sz["ff"], None, ff_act="silu"), SeqLayerSpec(att, 0, ex, ff_act="silu"),
+              SeqLayerSpec(lat, 0, ex, ff_act="silu"), SeqLayerSpec(att, 0, ex, ff_act="silu")]
+    cfg = SeqModelConfig("fepopel", sz["width"], SEQ_VOCAB, layers, name="fepopel-bench", block="sandwich",
+                         embed_scale=1.0, tied_head=False, loop=dict(FEP_LOOP))
+    cfg.validate()
+    return cfg
+
+
+def fep_kernel_rooflines(cfg, device, ctx, rows):
+    """The family's own kernels alone at `rows` token rows of one sequence that ends at position
+    ctx, as nab_kernel_rooflines reports them; `like` names the Naburax kernel each is set beside."""
+    from vllm_omni_draft_amd import ops
+    lat = next(l.mixer for l in cfg.layers if l.mixer.kind == "latent_attention")
+    att = next(l.mixer for l in cfg.layers if l.mixer.kind == "softmax_attention")
+    ex, W = cfg.layers[1].experts, cfg.width
+    g = torch.Generator(device="cpu").manual_seed(0)
+    rn = lambda *s: torch.randn(*s, generator=g).to(device)
+    pages = -(-ctx // ops.PAGE)
+    tables = torch.arange(pages, dtype=torch.int32, device=device).view(1, -1)
+    pos_l = list(range(ctx - rows, ctx))
+    pos = torch.tensor(pos_l, dtype=torch.int32, device=device)
+    slot = torch.zeros(rows, dtype=torch.int32, device=device)
+    out = []
+    # latent attention over every earlier token, with a sink: one cached row per token is key and value
+    H, de, rk = lat.heads, lat.kv_rank + lat.rot_dim, lat.kv_rank
+    keys = sum(p + 1 for p in pos_l)
+    kc = (torch.randn(pages, 1, ops.PAGE, de, generator=g) * 0.3).to(torch.bfloat16).to(device)
+    q, sinks = rn(rows, H * de), rn(H)
+    us = _events(lambda: ops.masked_softmax_attention(q, kc, None, pos, slot, tables, H, 1, de, rk, lat.scale,
+                                                      sinks=sinks), 5)
+    out.append(("masked_softmax_attention (latent rows, all keys, sink)", "window_softmax_attention (latent rows)", us,
+                2 * de * ctx + 4 * rows * H * (de + rk), 2.0 * keys * H * (de + rk), F32_VALU_PEAK_TFLOPS))
+    # grouped-query attention inside chunks, capped scores
+    H, G, D = att.heads, att.kv_heads, att.dim
+    keys = sum(p % att.chunk + 1 for p in pos_l)
+    span = min(ctx, max(p % att.chunk + 1 for p in pos_l) + rows - 1)
+    kc2 = torch.randn(pages, G, ops.PAGE, D, generator=g).to(torch.bfloat16).to(device)
+    vc2 = torch.randn(pages, G, ops.PAGE, D, generator=g).to(torch.bfloat16).to(device)
+    q2 = rn(rows, H * D)
+    us = _events(lambda: ops.masked_softmax_attention(q2, kc2, vc2, pos, slot, tables, H, G, D, D, att.scale,
+                                                      chunk=att.chunk, softcap=att.softcap), 5)
+    out.append(("masked_softmax_attention (grouped heads, chunks, cap)", "window_softmax_attention (grouped heads)", us,
+                G * 2 * D * 2 * span + 8 * rows * H * D, 2.0 * keys * H * 2 * D, F32_VALU_PEAK_TFLOPS))
+    # routed experts of two matrices (grouping, up, down)
+    E, top, F = ex.experts, ex.top, ex.ff
+    x = rn(rows, W)
+    up = (torch.randn(E, F, W, generator=g) * W ** -0.5).to(torch.bfloat16).to(device)
+    dn = (torch.randn(E, W, F, generator=g) * F ** -0.5).to(torch.bfloat16).to(device)
+    sel_e = torch.stack([torch.randperm(E, generator=g)[:top] for _ in range(rows)]).to(torch.int32).to(device)
+    sel_w = torch.rand(rows, top, generator=g).to(device)
+    us = _events(lambda: ops.moe_experts(x, sel_e, sel_w, up, dn, scale_input=False, act="relu2"), 5)
+    used = min(E, rows * top)
+    out.append(("moe_experts (two matrices)", "moe_experts", us,
+                2 * used * 2 * F * W + 4 * rows * W * (1 + top) + 2 * rows * top * F * 2,
+                2.0 * rows * top * 2 * F * W, BF16_MFMA_PEAK_TFLOPS))
+    # the router with its weights' scale and the shared expert's gate row
+    wr, wg = (torch.randn(E, W, generator=g) * W ** -0.5).to(torch.bfloat16).to(device), rn(1, W).to(torch.bfloat16)
+    us = _events(lambda: ops.moe_route_rows_gated(x, wr, top, "softmax", True, 1e-20, 1.5, wg), 5)
+    out.append(("moe_route_rows_gated", "moe_route_rows", us, 4 * rows * W + 2 * (E + 1) * W, 2.0 * rows * (E + 1) * W,
+                F32_VALU_PEAK_TFLOPS))
+    # residual update with the norms around it
+    a, b, gate = rn(rows * top, W), rn(rows, W), rn(rows, 1)
+    wp, wn = rn(W).to(torch.bfloat16), rn(W).to(torch.bfloat16)
+    xr = rn(rows, W)
+    us = _events(lambda: ops.residual_norm(xr, a, wp, top, b, gate, None, wn, 1e-5), 5)
+    out.append(("residual_norm", "postnorm_residual", us, 4 * rows * W * (top + 1 + 2 + 1) + 2 * rows * W, 0.0,
+                F32_VALU_PEAK_TFLOPS))
+    # Naburax's update, which norms the sublayer's output only, for comparison
+    us = _events(lambda: ops.postnorm_residual(xr, a, wp, 1e-5, n_a=top), 5)
+    out.append(("postnorm_residual (Naburax)", "", us, 4 * rows * W * (top + 2), 0.0, F32_VALU_PEAK_TFLOPS))
+    res = []
+    for name, like, us, nbytes, flops, peak in out:
+        floor_us = max(nbytes / (HBM_PEAK_GBS * 1e3), flops / (peak * 1e6))
+        res.append({"kernel": name, "like": like, "rows": rows, "ctx": ctx, "avg_us": round(us, 2),
+                    "min_bytes": int(nbytes), "flops": int(flops), "achieved_gbs": round(nbytes / us * 1e-3, 1),
+                    "achieved_tflops": round(flops / us * 1e-6, 2), "roofline_us": round(floor_us, 2),
+                    "times_roofline": round(us / floor_us, 1)})
+    return res
+
+
+def main_fep_family(args):
+    """Prefill and decode throughput of the Fepopel family beside the Naburax family at equal
+    width, heads and expert width (both bf16, seeded random weights), one JSON line."""
+    if not torch.cuda.is_available():
+        raise SystemExit("bench.py needs a GPU (there is no CPU path)")
+    device = torch.device("cuda", 0)
+    P, B, steps, warm = args.prompt_len, 4, args.steps, args.warmup
+    results = []
+    for name in args.seq_sizes.split(","):
+        sz = FEP_SIZES[name]
+        cfg = _fep_config(sz)
+        mine = _run_seq_engine(cfg, device, P, B, steps, warm)
+        mine["layer_runs"] = cfg.n_runs
+        kern = fep_kernel_rooflines(cfg, device, P, 1) + fep_kernel_rooflines(cfg, device, P, min(P, 1024))
+        ncfg = _nab_config(NAB_SIZES[name])
+        other = _run_seq_engine(ncfg, device, P, B, steps, warm)
+        other["layer_runs"] = ncfg.n_runs
+        like = nab_kernel_rooflines(ncfg, device, P, 1) + nab_kernel_rooflines(ncfg, device, P, min(P, 1024))
+        results.append({"size": name, **sz, "layers": [l.mixer.kind for l in cfg.layers], "loop": FEP_LOOP,
+                        "head_dim": SEQ_HEAD, "kv_rank": NAB_KV_RANK, "rot_dim": NAB_ROT, "chunk": FEP_CHUNK,
+                        "softcap": FEP_CAP, "prompt_len": P, "decode_batch": B, "fepopel": mine,
+                        "naburax_equal_size": other, "kernels": kern, "naburax_kernels": like})
+    print(json.dumps({"metric": "fepopel_family_throughput", "unit": "tokens/s", "dtype": "bf16",
+                      "data": "synthetic", "n_gpus": 1, "steps": steps, "warmup": warm, "sizes": results}))
+
 
 def main():
     args = parse()
+    if args.family == "fepopel":
+        main_fep_family(args)
+        return
     if args.family == "naburax":
         main_nab_family(args)
         return

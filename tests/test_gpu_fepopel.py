@@ -340,7 +340,7 @@ def test_experts_of_two_matrices(E, top, F, W, rows, wdt):
     assert rel(out, want) < (3e-6 if wdt == torch.float32 else 1e-2)
 
 
-@pytest.mark.parametrize("W", [5, 72, 1000])
+@pytest.mark.parametrize("W", [5, 72, 1000, 2048, 4100])
 def test_residual_update_and_following_norm(W):
     from vllm_omni_draft_amd import ops
     g = torch.Generator().manual_seed(W)

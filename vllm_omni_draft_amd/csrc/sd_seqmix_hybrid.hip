@@ -1264,6 +1264,7 @@ __global__ __launch_bounds__(256) void moe_down_mfma_kernel(
 // loads asked for before the first is used), then a butterfly sum.
 constexpr int kGemvMaxK = 8192;
 // act[a, n] (bf16) = silu(s * gate_e[n] . x) * (s * up_e[n] . x); wave: two columns, gate and up.
+// Not gated (an expert's first matrix alone, [F, K]): act[a, n] = relu(s * up_e[n] . x)^2; wave: four columns.
 template <bool GATED>
 __global__ __launch_bounds__(256) void moe_gemv_gate_up_kernel(
     const float* __restrict__ X, int64_t ldx, const int32_t* __restrict__ sel_e, const float* __restrict__ sel_w,
@@ -1273,13 +1274,22 @@ __global__ __launch_bounds__(256) void moe_gemv_gate_up_kernel(
   const float* xr = X + (size_t)(a / top) * ldx;
   for (int k = tid; k < K; k += 256) xs[k] = round_bf16(xr[k]);
   __syncthreads();
-  const int n0 = blockIdx.x * 8 + wave * 2;
+  constexpr int COLS = GATED ? 2 : 4;   // output columns of a wave: its four weight rows are gate, up of two, or four rows
+  const int n0 = (blockIdx.x * 4 + wave) * COLS;
   if (n0 >= F) return;
-  const int n1 = n0 + 1 < F ? n0 + 1 : n0;
-  // (not gated: an expert is one matrix [F, K]; the "up" rows alias the first, their sums go unused)
   const bf16_t* wg = Wgu + (size_t)e * (GATED ? 2 : 1) * F * K;
-  const bf16_t* wu = GATED ? wg + (size_t)F * K : wg;
-  const bf16_t* rows[4] = {wg + (size_t)n0 * K, wu + (size_t)n0 * K, wg + (size_t)n1 * K, wu + (size_t)n1 * K};
+  const bf16_t* rows[4];
+  if constexpr (GATED) {
+    const int n1 = n0 + 1 < F ? n0 + 1 : n0;
+    const bf16_t* wu = wg + (size_t)F * K;
+    rows[0] = wg + (size_t)n0 * K;
+    rows[1] = wu + (size_t)n0 * K;
+    rows[2] = wg + (size_t)n1 * K;
+    rows[3] = wu + (size_t)n1 * K;
+  } else {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) rows[j] = wg + (size_t)(n0 + j < F ? n0 + j : n0) * K;
+  }
   float acc[4] = {0.f, 0.f, 0.f, 0.f};
   for (int k0 = lane * 8; k0 < K; k0 += 4 * 512) {
     bf16x8 f[4][4];
@@ -1306,8 +1316,14 @@ __global__ __launch_bounds__(256) void moe_gemv_gate_up_kernel(
   for (int j = 0; j < 4; ++j) acc[j] = wave_sum(acc[j]);
   if (lane == 0) {
     const float sc = scale_input ? sel_w[a] : 1.f;
-    act[(size_t)a * F + n0] = (bf16_t)expert_act(sc * acc[0], sc * acc[1], GATED ? 0 : 1);
-    if (n0 + 1 < F) act[(size_t)a * F + n0 + 1] = (bf16_t)expert_act(sc * acc[2], sc * acc[3], GATED ? 0 : 1);
+    if constexpr (GATED) {
+      act[(size_t)a * F + n0] = (bf16_t)expert_act(sc * acc[0], sc * acc[1], 0);
+      if (n0 + 1 < F) act[(size_t)a * F + n0 + 1] = (bf16_t)expert_act(sc * acc[2], sc * acc[3], 0);
+    } else {
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        if (n0 + j < F) act[(size_t)a * F + n0 + j] = (bf16_t)expert_act(sc * acc[j], 0.f, 1);
+    }
   }
 }
 
@@ -1447,6 +1463,81 @@ __global__ __launch_bounds__(256) void residual_norm_kernel(
     const float v = maybe_round(row[c] * rstd2 * ld_f(w_next + c), round);
     if (h) h[(size_t)r * W + c] = v;
     if (h_b) h_b[(size_t)r * W + c] = (bf16_t)v;
+  }
+}
+
+// The same update four columns per thread (W a multiple of 4, rows 16-byte aligned), for up to
+// 1024 threads: a row of a few thousand columns is one or two pieces per thread, so every phase
+// waits for memory once.  Sums go lane -> wave -> workgroup in a fixed order.
+template <typename T> struct Quad;
+template <> struct Quad<float> {
+  static __device__ __forceinline__ f32x4 ld(const float* p) { return *reinterpret_cast<const f32x4*>(p); }
+};
+template <> struct Quad<bf16_t> {
+  static __device__ __forceinline__ f32x4 ld(const bf16_t* p) {
+    const bf16x4 v = *reinterpret_cast<const bf16x4*>(p);
+    return f32x4{(float)v[0], (float)v[1], (float)v[2], (float)v[3]};
+  }
+};
+__device__ __forceinline__ float block_sum_wide(float v, float* red) {   // up to 16 waves
+  v = wave_sum(v);
+  const int wave = threadIdx.x >> 6, n_waves = (blockDim.x + 63) >> 6;
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) red[wave] = v;
+  __syncthreads();
+  float s = red[0];
+  for (int w = 1; w < n_waves; ++w) s += red[w];
+  return s;
+}
+template <typename T>
+__global__ __launch_bounds__(1024) void residual_norm_quad_kernel(
+    float* __restrict__ x, const float* __restrict__ a, int n_a, const float* __restrict__ b,
+    const float* __restrict__ b_gate, int64_t ldg, const T* __restrict__ w_post, const T* __restrict__ add,
+    const T* __restrict__ w_next, float eps, float* __restrict__ x_copy, float* __restrict__ h,
+    bf16_t* __restrict__ h_b, int W, int round) {
+  extern __shared__ float row[];   // [W]
+  __shared__ float red[16];
+  const int r = blockIdx.x, nq = W / 4;
+  float rstd = 0.f;
+  if (a) {
+    const float gate = b ? (b_gate ? sigmoid_f(b_gate[(size_t)r * ldg]) : 1.f) : 0.f;
+    float ss = 0.f;
+    for (int c = threadIdx.x; c < nq; c += blockDim.x) {
+      f32x4 v = Quad<float>::ld(a + ((size_t)r * n_a) * W + 4 * c);
+      for (int j = 1; j < n_a; ++j) v += Quad<float>::ld(a + ((size_t)r * n_a + j) * W + 4 * c);
+      if (b) v += gate * Quad<float>::ld(b + (size_t)r * W + 4 * c);
+      *reinterpret_cast<f32x4*>(row + 4 * c) = v;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) ss = fmaf(v[i], v[i], ss);
+    }
+    ss = block_sum_wide(ss, red);
+    rstd = 1.f / sqrtf(ss / (float)W + eps);
+  }
+  float ss2 = 0.f;
+  for (int c = threadIdx.x; c < nq; c += blockDim.x) {
+    f32x4 xn = Quad<float>::ld(x + (size_t)r * W + 4 * c);
+    if (a) {
+      const f32x4 t = *reinterpret_cast<const f32x4*>(row + 4 * c), wp = Quad<T>::ld(w_post + 4 * c);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) xn[i] += t[i] * rstd * wp[i];
+    }
+    if (x_copy) *reinterpret_cast<f32x4*>(x_copy + (size_t)r * W + 4 * c) = xn;
+    if (add) xn += Quad<T>::ld(add + 4 * c);
+    if (a || add) *reinterpret_cast<f32x4*>(x + (size_t)r * W + 4 * c) = xn;
+    *reinterpret_cast<f32x4*>(row + 4 * c) = xn;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) ss2 = fmaf(xn[i], xn[i], ss2);
+  }
+  if (!w_next) return;
+  ss2 = block_sum_wide(ss2, red);
+  const float rstd2 = 1.f / sqrtf(ss2 / (float)W + eps);
+  for (int c = threadIdx.x; c < nq; c += blockDim.x) {
+    const f32x4 xn = *reinterpret_cast<const f32x4*>(row + 4 * c), wn = Quad<T>::ld(w_next + 4 * c);
+    f32x4 v;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v[i] = maybe_round(xn[i] * rstd2 * wn[i], round);
+    if (h) *reinterpret_cast<f32x4*>(h + (size_t)r * W + 4 * c) = v;
+    if (h_b) *reinterpret_cast<bf16x4*>(h_b + (size_t)r * W + 4 * c) = bf16x4{(bf16_t)v[0], (bf16_t)v[1], (bf16_t)v[2], (bf16_t)v[3]};
   }
 }
 
@@ -1885,7 +1976,7 @@ extern "C" int sd_moe_experts(const float* x, const void* x_bf16, int64_t ldx, c
       moe_gemv_gate_up_kernel<true><<<dim3((F + 7) / 8, n), 256, sizeof(float) * W, st>>>(
           x, ldx, sel_expert, sel_weight, (const bf16_t*)w_gate_up, act_b, top, F, W, scale_input);
     else
-      moe_gemv_gate_up_kernel<false><<<dim3((F + 7) / 8, n), 256, sizeof(float) * W, st>>>(
+      moe_gemv_gate_up_kernel<false><<<dim3((F + 15) / 16, n), 256, sizeof(float) * W, st>>>(
           x, ldx, sel_expert, sel_weight, (const bf16_t*)w_gate_up, act_b, top, F, W, scale_input);
     SD_CHECK_LAUNCH("sd_moe_experts (gate, up)");
     moe_gemv_down_kernel<<<dim3((W + 15) / 16, n), 256, sizeof(float) * F, st>>>(
@@ -1936,6 +2027,24 @@ extern "C" int sd_residual_norm(float* x, const float* a, int n_a, const float* 
   SD_REQUIRE((size_t)W * sizeof(float) <= 60 * 1024, SD_ERR_UNSUPPORTED, "sd_residual_norm: width %d above 15360", W);
   hipStream_t st = (hipStream_t)stream;
   const size_t lds = (size_t)W * sizeof(float);
+  auto al16 = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
+  // (weights are 4 or 2 bytes an element: four of them are 16 or 8 bytes, and a vector [W] starts aligned to that
+  // when its address is a multiple of 16; `add` may be a row of a table, whose rows are W elements apart)
+  if (W % 4 == 0 && W >= 256 && al16(x) && al16(a) && al16(b) && al16(w_post) && al16(w_next) && al16(x_copy) &&
+      al16(h) && al16(h_bf16) && (reinterpret_cast<uintptr_t>(add) & 7) == 0 && (!w_f32 || al16(add))) {
+    int nthr = ((W / 4 + 63) / 64) * 64;
+    if (nthr > 1024) nthr = 1024;
+    if (w_f32)
+      residual_norm_quad_kernel<float><<<n_rows, nthr, lds, st>>>(x, a, n_a, b, b_gate, ldg, (const float*)w_post,
+                                                                  (const float*)add, (const float*)w_next, eps, x_copy,
+                                                                  h, (bf16_t*)h_bf16, W, 0);
+    else
+      residual_norm_quad_kernel<bf16_t><<<n_rows, nthr, lds, st>>>(x, a, n_a, b, b_gate, ldg, (const bf16_t*)w_post,
+                                                                   (const bf16_t*)add, (const bf16_t*)w_next, eps,
+                                                                   x_copy, h, (bf16_t*)h_bf16, W, 1);
+    SD_CHECK_LAUNCH("sd_residual_norm");
+    return SD_OK;
+  }
   if (w_f32)
     residual_norm_kernel<float><<<n_rows, 256, lds, st>>>(x, a, n_a, b, b_gate, ldg, (const float*)w_post,
                                                           (const float*)add, (const float*)w_next, eps, x_copy, h,
