@@ -583,6 +583,8 @@ def naburax_config(cfg: dict, tensor_shapes: Optional[dict] = None, **overrides)
                              rot_dims=int(rot.get("dims", 0)), rot_base=float(rot.get("base", 10000.0)),
                              rot_layout="interleaved", rot_scaling=rot.get("scaling") or None,
                              scale=float(m["scale"]), window=int(m["mask"]["size"]))
+            if spec.q_rank < 1 or spec.window < 1:
+                raise ValueError(f"layer {i}: latent attention needs a query latent and a window of at least one token")
         elif kind == "parallel":
             a, b = m["left"], m["right"]
             spec = MixerSpec(kind=kind, heads=int(a["heads"]), kv_heads=int(a.get("kv_heads", 0)), dim=int(a["dim"]),

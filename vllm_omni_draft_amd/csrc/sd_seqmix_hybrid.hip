@@ -382,25 +382,48 @@ __global__ __launch_bounds__(256) void window_softmax_attn_kernel(
   }
 }
 
-// out[r, h] = sum_s acc_s exp(m_s - M) / sum_s l_s exp(m_s - M), tiles s in order, M = max m_s.
+// out[r, h] = sum_s acc_s exp(m_s - M) / sum_s l_s exp(m_s - M), M = max m_s.  The first wave takes
+// the tiles' maxima and sums a lane per tile (butterfly sums: a fixed order) and leaves every
+// tile's factor in LDS; then a thread per column adds the tiles' rows in tile order, eight loads
+// in flight.
 __global__ void softmax_merge_kernel(const float* __restrict__ part_acc, const float* __restrict__ part_ml,
                                      int n_splits, float* __restrict__ out, bf16_t* __restrict__ out_b, int H, int dv) {
-  const int r = blockIdx.x, h = blockIdx.y, R = gridDim.x;
-  float M = -INFINITY;
-  for (int s = 0; s < n_splits; ++s) M = fmaxf(M, part_ml[(((size_t)s * R + r) * H + h) * 2]);
-  float L = 0.f;
-  for (int s = 0; s < n_splits; ++s) {
-    const float* ml = part_ml + (((size_t)s * R + r) * H + h) * 2;
-    if (ml[0] != -INFINITY) L += ml[1] * expf(ml[0] - M);
-  }
-  for (int c = threadIdx.x; c < dv; c += blockDim.x) {
-    float o = 0.f;
-    for (int s = 0; s < n_splits; ++s) {
-      const float m = part_ml[(((size_t)s * R + r) * H + h) * 2];
-      if (m != -INFINITY) o = fmaf(part_acc[(((size_t)s * R + r) * H + h) * dv + c], expf(m - M), o);
+  extern __shared__ float fac[];   // [n_splits]
+  __shared__ float inv_l;
+  const int r = blockIdx.x, h = blockIdx.y, R = gridDim.x, tid = threadIdx.x;
+  const size_t stride = (size_t)R * H;             // (row, head) pairs of one tile
+  const size_t at0 = (size_t)r * H + h;
+  if (tid < 64) {
+    float M = -INFINITY;
+    for (int s = tid; s < n_splits; s += 64) M = fmaxf(M, part_ml[(s * stride + at0) * 2]);
+    M = wave_max(M);
+    float L = 0.f;
+    for (int s = tid; s < n_splits; s += 64) {
+      const float* ml = part_ml + (s * stride + at0) * 2;
+      const float f = ml[0] == -INFINITY ? 0.f : expf(ml[0] - M);
+      fac[s] = f;
+      L += ml[1] * f;
     }
-    o /= L;
-    const size_t at = ((size_t)r * H + h) * dv + c;
+    L = wave_sum(L);
+    if (tid == 0) inv_l = 1.f / L;
+  }
+  __syncthreads();
+  constexpr int kU = 8;
+  for (int c = tid; c < dv; c += blockDim.x) {
+    float o = 0.f;
+    for (int s0 = 0; s0 < n_splits; s0 += kU) {
+      float v[kU];
+#pragma unroll
+      for (int u = 0; u < kU; ++u) {
+        const int s = s0 + u < n_splits ? s0 + u : n_splits - 1;
+        v[u] = part_acc[(s * stride + at0) * dv + c];
+      }
+#pragma unroll
+      for (int u = 0; u < kU; ++u)
+        if (s0 + u < n_splits && fac[s0 + u] != 0.f) o = fmaf(v[u], fac[s0 + u], o);
+    }
+    o *= inv_l;
+    const size_t at = at0 * dv + c;
     out[at] = o;
     if (out_b) out_b[at] = (bf16_t)o;
   }
@@ -1785,7 +1808,7 @@ extern "C" int sd_masked_softmax_attention(const float* q, int64_t ldq, const vo
 #undef SD_NH
   SD_CHECK_LAUNCH("sd_masked_softmax_attention");
   if (split) {
-    softmax_merge_kernel<<<dim3(n_rows, H), dv <= 64 ? 64 : (dv <= 128 ? 128 : 256), 0, st>>>(
+    softmax_merge_kernel<<<dim3(n_rows, H), dv <= 64 ? 64 : (dv <= 128 ? 128 : 256), sizeof(float) * n_splits, st>>>(
         part_acc, part_ml, n_splits, out, (bf16_t*)out_bf16, H, dv);
     SD_CHECK_LAUNCH("sd_masked_softmax_attention (merge)");
   }

@@ -275,6 +275,13 @@ class SeqWorker:
                                                          max_seq_len=c.max_model_len))
 
     def _sample(self, logits: torch.Tensor, rids: List[str]) -> List[int]:
+        V = logits.shape[1]
+        if V % 4:
+            # the sampling kernels read rows in 16-byte pieces: a vocabulary that is no multiple of
+            # four is padded with columns that can never be chosen
+            wide = torch.full((logits.shape[0], V + 4 - V % 4), float("-inf"), dtype=torch.float32, device=logits.device)
+            wide[:, :V] = logits
+            return [min(t, V - 1) for t in self._sample(wide, rids)]
         reqs = [self._req[r] for r in rids]
         temps = [r["sp"].temperature or 0.0 for r in reqs]
         if not any(t > 0 for t in temps):
