@@ -46,7 +46,7 @@ def draw_model(rng):
 
     n = rng.randint(1, 6)
     layers = [rng.choice([latent, latent, chunked])() for _ in range(n)]
-    cfg = {"architecture": "Fepopel", "width": rng.choice([24, 40, 56, 64, 72, 96, 128, 160]),
+    cfg = {"architecture": "Fepopel", "width": rng.choice([24, 40, 56, 64, 72, 96, 128, 160, 256, 320, 516]),
            "vocab": rng.randint(40, 700), "norm": {"eps": rng.choice([1e-5, 1e-6])},
            "embedding": {"scale": rng.choice([1.0, 3.0, 12.0])}, "layers": layers}
     if rng.random() < 0.8:

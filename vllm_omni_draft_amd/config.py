@@ -640,7 +640,7 @@ def fepopel_config(cfg: dict, tensor_shapes: Optional[dict] = None, **overrides)
             mask = m.get("mask") or {}
             spec = MixerSpec(kind="softmax_attention", heads=int(m["heads"]), kv_heads=int(m.get("kv_heads", 0)),
                              dim=int(m["dim"]), vdim=int(m["vdim"]), scale=float(m["scale"]), window=0,
-                             chunk=int(mask.get("size", 0)), softcap=float(m.get("softcap", 0.0)), qk_head_norm=True)
+                             chunk=int(mask.get("size") or 0), softcap=float(m.get("softcap") or 0.0), qk_head_norm=True)
         else:
             raise ValueError(f"layer {i}: unknown mixer type {kind!r}")
         mlp = l.get("mlp")
