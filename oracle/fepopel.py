@@ -51,7 +51,8 @@ def attend(q, k, v, pos_q, scale, chunk=0, softcap=0.0, sink=None):
     s = torch.einsum("ihd,jhd->hij", q.to(F64), k) * scale
     if softcap > 0:
         s = softcap * torch.tanh(s / softcap)
-    seen = torch.tensor([[visible(int(i), j, chunk) for j in range(T)] for i in pos_q])
+    i, j = torch.as_tensor(pos_q).long()[:, None], torch.arange(T)[None, :]
+    seen = (j <= i) & ((i // chunk == j // chunk) if chunk > 0 else True)          # visible(i, j, chunk), all pairs at once
     s = s.masked_fill(~seen[None], -math.inf)
     mx = s.max(-1).values
     if sink is not None:

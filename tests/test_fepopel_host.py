@@ -35,6 +35,11 @@ def test_chunk_rule():
             seen = [j for j in range(25) if P.visible(i, j, chunk)]
             lo = 0 if chunk == 0 else i - i % chunk
             assert seen == list(range(lo, i + 1))
+        # the attention of the plain model applies the same rule: one-hot values show who is seen
+        q, k, v = torch.zeros(20, 1, 2, dtype=torch.float64), torch.zeros(25, 1, 2, dtype=torch.float64), torch.eye(25, dtype=torch.float64)[:, None, :]
+        w = P.attend(q, k, v, list(range(20)), 1.0, chunk=chunk)[:, 0]
+        for i in range(20):
+            assert [j for j in range(25) if w[i, j] > 0] == [j for j in range(25) if P.visible(i, j, chunk)]
 
 
 def test_order_of_running():
