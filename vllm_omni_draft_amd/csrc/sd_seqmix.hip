@@ -1025,7 +1025,6 @@ SwCols sw_cols(const sd_seq_layer& l) {
   return c;
 }
 inline int act_inputs(int act_kind) { return act_kind == 2 ? 1 : 2; }   // matrices an activation of sd_act_rows reads
-constexpr int kNoWindow = 0x7fffffff;
 PnCols pn_cols(const sd_seq_layer& l) {
   PnCols c = {};
   int at = 0;
