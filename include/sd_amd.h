@@ -1295,6 +1295,57 @@ int sd_residual_norm(float* x, const float* a, int n_a, const float* b, const fl
                      int64_t ldg, const void* w_post, const void* add, const void* w_next,
                      int w_f32, float eps, float* x_copy, float* h, void* h_bf16, int n_rows,
                      int W, sd_stream_t stream);
+/* sd_masked_softmax_attention with `maps` score maps per head: q [rows, H*maps*dk], head h's map m
+ * at channel (h*maps + m)*dk; the key cache holds `maps` key rows per kv head and token (cache head
+ * g*maps + m, as sd_attn_prep appends them), the value cache one row per kv head, which every map
+ * of the heads of that kv head reads.  out [rows, H*maps, dv]: every map's own softmax-weighted
+ * values; sinks (or NULL) f32 [H*maps].  maps == 1: sd_masked_softmax_attention itself.        */
+size_t sd_multimap_softmax_attention_scratch_bytes(int n_rows, int H, int maps, int dv, int window,
+                                                   int keep_first, int chunk, int max_ctx);
+int sd_multimap_softmax_attention(const float* q, int64_t ldq, const void* k_cache,
+                                  const void* v_cache, int cache_f32, const int32_t* row_pos,
+                                  const int32_t* row_slot, const int32_t* block_tables,
+                                  int max_blocks, int page, int n_rows, int H, int G, int maps, int dk,
+                                  int dv, int window, int keep_first, int chunk, float scale,
+                                  float softcap, const float* sinks, float* out, void* out_bf16,
+                                  void* scratch, size_t scratch_bytes, sd_stream_t stream);
+/* Grouped-query attention's preparation in one launch, in place on q [rows, n_q_units*dk] and
+ * k [rows, n_k_units*dk] (row stride ld; a unit is one head's one score map): + q_bias / k_bias
+ * (model element type, or NULL); norm_kind 1: RMS norm over the whole row times q_norm_w
+ * [n_q_units*dk] / k_norm_w [n_k_units*dk]; 2: per unit, times one weight [dk]; 0: none; then
+ * every unit's first rot_dims channels turned as sd_rope_rows does.  The keys are appended to
+ * k_cache (cache head = unit) and the values v [rows, G*dv] to v_cache as sd_cache_append does;
+ * value_from_key: there is no v, and a value row is the key row after its bias, before norm and
+ * turn (G*dv == n_k_units*dk).  k == NULL: only q is prepared (a layer that reads the keys and
+ * values another layer appended).                                                          */
+int sd_attn_prep(float* q, int n_q_units, float* k, int n_k_units, int dk, const float* v, int G,
+                 int dv, int value_from_key, int64_t ld, const void* q_bias, const void* k_bias,
+                 int norm_kind, const void* q_norm_w, const void* k_norm_w, int w_f32, float eps,
+                 int rot_dims, int rot_layout, const double* inv_freq, float mag, void* k_cache,
+                 void* v_cache, const int32_t* row_pos, const int32_t* row_slot,
+                 const int32_t* block_tables, int max_blocks, int page, int n_rows,
+                 sd_stream_t stream);
+/* Differential attention's last step: a [rows, H, 2, dv] holds two maps' outputs per head;
+ * y[r, h] = t / sqrt(mean(t^2) + eps) * out_scale with t = a[r, h, 0] - lambda * a[r, h, 1], the
+ * mean over the head's dv channels.  y [rows, H*dv]; y_bf16 (or NULL) the same as bf16.        */
+int sd_diff_combine_rows(const float* a, float lambda, float eps, float out_scale, float* y,
+                         void* y_bf16, int n_rows, int H, int dv, int round_bf16_out,
+                         sd_stream_t stream);
+/* sd_moe_route_rows_gated with router_bias (f32 [E], or NULL) added to the router's logits
+ * before anything is chosen.                                                                */
+int sd_moe_route_rows_biased(const float* x, int64_t ldx, const void* w_router,
+                             const float* router_bias, int w_f32, float* logits,
+                             int32_t* sel_expert, float* sel_weight, int n_rows, int E, int K, int top,
+                             int score_kind, int renorm, float renorm_eps, float weight_scale,
+                             const void* w_gate, int n_gate, float* gate_out, sd_stream_t stream);
+/* sd_residual_norm with a_bias ([W], model element type, or NULL) added to the sum t before its
+ * norm (the bias of the sublayer's output matrix), and the update multiplied by mult:
+ * x[r] += mult * rms_norm(t) * w_post.                                                       */
+int sd_residual_norm_scaled(float* x, const float* a, int n_a, const void* a_bias, const float* b,
+                            const float* b_gate, int64_t ldg, const void* w_post, float mult,
+                            const void* add, const void* w_next, int w_f32, float eps,
+                            float* x_copy, float* h, void* h_bf16, int n_rows, int W,
+                            sd_stream_t stream);
 /* x[r, c] *= s                                                                             */
 int sd_scale_rows(float* x, int64_t ld, float s, int n_rows, int n_cols, sd_stream_t stream);
 
@@ -1414,6 +1465,21 @@ typedef struct {
   const void* w_shared_down; /* [width, shared_ff] */
   const void* w_shared_down_tiled;
   const void* w_shared_gate; /* [1, width] or NULL: no gate */
+  /* ---- SD_MIX_SOFTMAX in general (all zero: as above).  w_in stacks q [heads*maps*dim], then,
+   * unless kv_shared, k [kv_heads*maps*dim], then, unless kv_shared or value_from_key, v
+   * [kv_heads*vdim].  rot_dims / rot_layout / inv_freq / rot_mag turn q and k; sinks may be given. */
+  int maps;                 /* score maps per head (0 or 1: one).  2: differential attention, a head's
+                               output is map 0's minus diff_lambda times map 1's, divided by its root
+                               mean square, times diff_scale */
+  float diff_lambda, diff_scale;
+  int qk_full_norm;         /* q_norm_w [heads*maps*dim] / k_norm_w [kv_heads*maps*dim] norm the whole projection */
+  int value_from_key;       /* a value row is the key row as projected (after its bias): vdim == dim */
+  int kv_shared;            /* k_cache / v_cache belong to an earlier layer of the same head layout,
+                               which has appended this pass's rows already */
+  const void* w_in_bias;    /* [w_in's rows] (model element type) or NULL: biases of q and k */
+  const void* w_o_bias;     /* [width] or NULL */
+  const float* router_bias; /* f32 [n_experts] or NULL */
+  float residual_mult;      /* factor of both residual updates; 0: 1 */
 } sd_seq_layer;
 
 typedef struct {

@@ -99,7 +99,10 @@ class SeqLayer(C.Structure):
                 ("ff_act", i32), ("expert_act", i32), ("route_score", i32), ("route_renorm", i32),
                 ("expert_scale_input", i32), ("route_renorm_eps", C.c_float), ("route_scale", C.c_float),
                 ("shared_ff", i32), ("shared_act", i32), ("w_shared_in", vp), ("w_shared_in_tiled", vp),
-                ("w_shared_down", vp), ("w_shared_down_tiled", vp), ("w_shared_gate", vp)]
+                ("w_shared_down", vp), ("w_shared_down_tiled", vp), ("w_shared_gate", vp),
+                ("maps", i32), ("diff_lambda", C.c_float), ("diff_scale", C.c_float), ("qk_full_norm", i32),
+                ("value_from_key", i32), ("kv_shared", i32), ("w_in_bias", vp), ("w_o_bias", vp),
+                ("router_bias", vp), ("residual_mult", C.c_float)]
 
 
 class SeqModelDesc(C.Structure):
@@ -274,6 +277,16 @@ SIGNATURES = {
     "sd_moe_route_rows_gated": (i32, [vp, i64, vp, i32, vp, vp, vp, i32, i32, i32, i32, i32, i32, C.c_float, C.c_float,
                                       vp, i32, vp, vp]),
     "sd_residual_norm": (i32, [vp, vp, i32, vp, vp, i64, vp, vp, vp, i32, C.c_float, vp, vp, vp, i32, i32, vp]),
+    "sd_multimap_softmax_attention_scratch_bytes": (C.c_size_t, [i32, i32, i32, i32, i32, i32, i32, i32]),
+    "sd_multimap_softmax_attention": (i32, [vp, i64, vp, vp, i32, vp, vp, vp, i32, i32, i32, i32, i32, i32, i32, i32,
+                                            i32, i32, i32, C.c_float, C.c_float, vp, vp, vp, vp, C.c_size_t, vp]),
+    "sd_attn_prep": (i32, [vp, i32, vp, i32, i32, vp, i32, i32, i32, i64, vp, vp, i32, vp, vp, i32, C.c_float, i32,
+                           i32, vp, C.c_float, vp, vp, vp, vp, vp, i32, i32, i32, vp]),
+    "sd_diff_combine_rows": (i32, [vp, C.c_float, C.c_float, C.c_float, vp, vp, i32, i32, i32, i32, vp]),
+    "sd_moe_route_rows_biased": (i32, [vp, i64, vp, vp, i32, vp, vp, vp, i32, i32, i32, i32, i32, i32, C.c_float,
+                                       C.c_float, vp, i32, vp, vp]),
+    "sd_residual_norm_scaled": (i32, [vp, vp, i32, vp, vp, vp, i64, vp, C.c_float, vp, vp, i32, C.c_float, vp, vp,
+                                      vp, i32, i32, vp]),
     "sd_seq_model_create": (vp, [C.POINTER(SeqModelDesc)]),
     "sd_seq_model_destroy": (None, [vp]),
     "sd_seq_model_workspace_bytes": (C.c_size_t, [vp, i32, i32, i32]),

@@ -250,7 +250,8 @@ class ExpertsSpec:
     (else its output).  act "silu": an expert is down(silu(gate h) * (up h)); "relu2": an expert has
     two matrices, down(relu(up h)^2).  The chosen weights are divided by (their sum + renorm_eps)
     when renorm, then multiplied by scale.  shared_ff > 0: one more expert of that width and the
-    same form runs for every token and is added, times sigmoid(g . h) when shared_gate."""
+    same form runs for every token and is added, times sigmoid(g . h) when shared_gate.  A softmax
+    score that is renormed over the chosen experts is the softmax over the chosen logits alone."""
     experts: int
     top: int
     ff: int
@@ -262,6 +263,7 @@ class ExpertsSpec:
     scale: float = 1.0
     shared_ff: int = 0
     shared_gate: bool = True
+    router_bias: bool = False      # a bias on the router's logits
 
     def validate(self) -> None:
         if self.experts < 1 or not 1 <= self.top <= self.experts or self.ff < 1 or self.shared_ff < 0:
@@ -290,7 +292,15 @@ class MixerSpec:
     tanh(s / softcap), keys of the query's own chunk of `chunk` positions only.  A latent
     attention with q_rank 0 projects its queries straight from the input; window 0 sees every
     earlier token; sink: a learned term per head in the softmax's denominator; head_gate: a
-    head's output is multiplied by the sigmoid of a product of the input."""
+    head's output is multiplied by the sigmoid of a product of the input.  A softmax attention
+    may also: rotate the leading rot_dims channels of q and k (rot_layout, rot_base, rot_scaling);
+    hold `maps` score maps per head over the same values (2: differential attention, map 0's output
+    minus lambda times map 1's, the difference divided by its root mean square and multiplied by
+    1 - diff; lambda = exp(lq1 . lk1) - exp(lq2 . lk2) + diff from four learned vectors); norm q and
+    k over the whole projection (qk_full_norm); add biases to the q, k and output projections
+    (proj_bias); take its values from the keys as projected (value_is_key: no value matrix); keep
+    one term of score 0 in the softmax's denominator (unit_sink); read the keys and values that
+    layer kv_from cached instead of projecting its own."""
     kind: str
     heads: int
     dim: int
@@ -318,6 +328,13 @@ class MixerSpec:
     sink: bool = False             # a learned term per head in the softmax's denominator
     head_gate: bool = False        # outputs gated per head
     qk_head_norm: bool = False     # q and k normed per head
+    maps: int = 1                  # softmax attention: score maps per head
+    diff: float = 0.0              # differential attention's constant
+    qk_full_norm: bool = False     # q and k normed over the whole projection
+    proj_bias: bool = False        # biases on the q, k and output projections
+    value_is_key: bool = False     # values are the keys as projected
+    unit_sink: bool = False        # one term exp(0) in the softmax's denominator
+    kv_from: int = -1              # the layer whose cached keys and values this one reads (-1: its own)
 
     def validate(self) -> None:
         if self.kind not in MIXER_KINDS:
@@ -337,8 +354,14 @@ class MixerSpec:
                 raise ValueError("latent attention: kv_rank above 512, or kv_heads given")
             return
         if self.kind == "softmax_attention":
-            if self.window < 0 or self.chunk < 0 or self.softcap < 0 or self.rot_dims or self.vdim > 512:
-                raise ValueError("softmax attention needs window >= 0, chunk >= 0, softcap >= 0, no rotation, vdim <= 512")
+            if self.window < 0 or self.chunk < 0 or self.softcap < 0 or self.vdim > 512:
+                raise ValueError("softmax attention needs window >= 0, chunk >= 0, softcap >= 0, vdim <= 512")
+            if self.rot_dims < 0 or self.rot_dims % 2 or self.rot_dims > self.dim:
+                raise ValueError(f"rot_dims {self.rot_dims} must be even and at most dim {self.dim}")
+            if self.maps not in (1, 2) or (self.qk_head_norm and self.qk_full_norm) or (self.sink and self.unit_sink):
+                raise ValueError("softmax attention: one or two score maps, one kind of q/k norm, one kind of sink")
+            if self.value_is_key and (self.maps != 1 or self.vdim != self.dim or self.kv_from >= 0):
+                raise ValueError("values taken from the keys need one score map, vdim == dim and keys of the layer's own")
             return
         if self.kind == "parallel":
             if self.window < 1 or self.keep_first < 0 or self.rot_dims or self.ssd is None or self.vdim > 512:
@@ -371,11 +394,13 @@ def rotary_frequencies(dims: int, base: float, scaling: Optional[dict] = None):
     and 1.  With scaling {factor, original, fast, slow}: pair i keeps its frequency f_i where it
     turns fast and takes f_i / factor where it turns slowly, blended along a ramp over the pair
     index between the pairs that make `fast` and `slow` turns over `original` positions; cos and
-    sin grow by 0.1 ln(factor) + 1."""
+    sin grow by 0.1 ln(factor) + 1.  With scaling {factor} alone every frequency is f_i / factor."""
     i = torch.arange(dims // 2, dtype=torch.float64)
     f = torch.tensor(float(base), dtype=torch.float64) ** (-2.0 * i / dims)
     if not scaling:
         return f, 1.0
+    if "original" not in scaling:
+        return f / float(scaling["factor"]), 1.0
     factor, orig = float(scaling["factor"]), float(scaling["original"])
 
     def pair_index(turns: float) -> float:
@@ -419,6 +444,7 @@ class SeqModelConfig:
     # (every pass keeps a cache of its own); the learned vector 'loop.step'[t] is added to the
     # stream before pass t.
     loop: Optional[dict] = None
+    residual_mult: float = 1.0     # "sandwich": both residual updates are multiplied by it
 
     @property
     def runs(self) -> List[tuple]:
@@ -435,14 +461,23 @@ class SeqModelConfig:
         return len(self.runs)
 
     def _validate_sandwich(self) -> None:
-        for l in self.layers:
+        for i, l in enumerate(self.layers):
             l.mixer.validate()
             if l.mixer.kind not in ("latent_attention", "softmax_attention"):
                 raise ValueError(f"mixer {l.mixer.kind!r} does not belong to a 'sandwich' model")
             if l.mixer.kind == "latent_attention" and l.mixer.q_rank:
                 raise ValueError("a 'sandwich' model's latent attention projects its queries straight from the input")
-            if l.mixer.kind == "softmax_attention" and not l.mixer.qk_head_norm:
-                raise ValueError("a 'sandwich' model's softmax attention norms q and k per head")
+            src = l.mixer.kv_from
+            if src >= 0:
+                if self.loop is not None or l.mixer.kind != "softmax_attention" or not src < i:
+                    raise ValueError(f"layer {i}: keys and values are read from an earlier softmax attention layer "
+                                     "of a model without a repeated span")
+                a, b = l.mixer, self.layers[src].mixer
+                same = ("kind", "heads", "kv_heads", "dim", "vdim", "maps", "rot_dims", "rot_base", "rot_layout",
+                        "rot_scaling", "qk_head_norm", "qk_full_norm")
+                if b.kv_from >= 0 or b.value_is_key or any(getattr(a, k) != getattr(b, k) for k in same):
+                    raise ValueError(f"layer {i}: layer {src} must project keys and values of its own, with this "
+                                     "layer's head counts, sizes, norms and rotation")
             if l.ff < 0 or l.ff_act not in ("relu", "silu") or (l.ff and l.experts is not None):
                 raise ValueError("a layer's feed-forward is gated (ff > 0, relu or silu) or routed experts, not both")
             if l.experts is not None:
@@ -499,13 +534,19 @@ class SeqModelConfig:
                     n += W * (m.heads * (m.dim + m.rot_dim) + m.kv_rank + m.rot_dim + (m.heads if m.head_gate else 0))
                     n += m.kv_rank + m.heads * (m.dim + m.vdim) * m.kv_rank + (m.heads if m.sink else 0)
                 else:
-                    n += W * (m.heads * m.dim + m.kv_heads * (m.dim + m.vdim)) + 2 * m.dim
+                    nq, nk = m.heads * m.maps * m.dim, m.kv_heads * m.maps * m.dim
+                    nv = 0 if m.value_is_key else m.kv_heads * m.vdim
+                    n += W * nq + (0 if m.kv_from >= 0 else W * (nk + nv))
+                    n += 2 * m.dim if m.qk_head_norm else ((nq + nk) if m.qk_full_norm else 0)
+                    n += (nq + nk + W) if m.proj_bias else 0
+                    n += 4 * m.dim if m.maps == 2 else 0
                 n += 3 * l.ff * W
                 ex = l.experts
                 if ex is not None:
                     per = 3 if ex.act == "silu" else 2
                     n += ex.experts * (W + per * ex.ff * W) + per * ex.shared_ff * W
                     n += W if ex.shared_ff and ex.shared_gate else 0
+                    n += ex.experts if ex.router_bias else 0
                 continue
             if m.kind == "latent_attention":
                 n += W + W * (m.q_rank + m.kv_rank + m.rot_dim) + m.q_rank + m.kv_rank
@@ -670,8 +711,55 @@ def fepopel_config(cfg: dict, tensor_shapes: Optional[dict] = None, **overrides)
     return out
 
 
+def zopupel_config(cfg: dict, tensor_shapes: Optional[dict] = None, **overrides) -> SeqModelConfig:
+    """A Zopupel config.json: layers normed before and after each sublayer, both residual updates
+    multiplied by one constant; two causal grouped-query softmax attentions over every earlier
+    token, in any order, with rotate-half rotary positions on the leading channels: "attention", a
+    differential attention (two score maps per head, every frequency divided by a factor), which
+    may read an earlier layer's cached keys and values (kv_from); "attention_2", whose values are
+    its keys as projected, with biases on its projections, q and k normed over the whole
+    projection, blended frequencies and one term of score 0 in the softmax's denominator.  Routed
+    gated experts (a bias on the router, softmax over the chosen logits) beside an ungated shared
+    expert, or no feed-forward; an untied head."""
+    layers = []
+    for i, l in enumerate(cfg["layers"]):
+        m, kind = l["mixer"], l["type"]
+        rot = m.get("rot") or {}
+        common = dict(kind="softmax_attention", heads=int(m["heads"]), kv_heads=int(m.get("kv_heads", 0)),
+                      dim=int(m["dim"]), vdim=int(m["vdim"]), scale=float(m["scale"]), window=0,
+                      rot_dims=int(rot.get("dims", 0)), rot_base=float(rot.get("base", 10000.0)), rot_layout="half",
+                      rot_scaling=rot.get("scaling") or None)
+        if kind == "attention":
+            src = m.get("kv_from")
+            spec = MixerSpec(maps=2, diff=float(m["diff"]), kv_from=-1 if src is None else int(src), **common)
+        elif kind == "attention_2":
+            spec = MixerSpec(qk_full_norm=True, proj_bias=True, value_is_key=True, unit_sink=True, **common)
+        else:
+            raise ValueError(f"layer {i}: unknown mixer type {kind!r}")
+        mlp = l.get("mlp")
+        experts = None
+        if mlp:
+            if mlp.get("kind", "moe") != "moe":
+                raise ValueError(f"layer {i}: feed-forward kind {mlp.get('kind')!r} is not supported")
+            r, sh = mlp["router"], mlp.get("shared")
+            experts = ExpertsSpec(experts=int(r["experts"]), top=int(r["top"]), ff=int(mlp["expert"]["ff"]),
+                                  score="softmax", renorm=True, scale_input=False, act="silu",
+                                  shared_ff=int(sh["ff"]) if sh else 0, shared_gate=False, router_bias=True)
+        layers.append(SeqLayerSpec(spec, 0, experts, ff_act="silu"))
+    out = SeqModelConfig(arch="zopupel", width=int(cfg["width"]), vocab=int(cfg["vocab"]), layers=layers,
+                         norm_eps=float(cfg["norm"]["eps"]), name=cfg.get("architecture", "Zopupel"),
+                         block="sandwich", tied_head=False, residual_mult=float(cfg.get("residual_mult", 1.0)))
+    for k, v in overrides.items():
+        if not hasattr(out, k):
+            raise ValueError(f"Unknown config parameter: {k}")
+        setattr(out, k, v)
+    out.validate()
+    return out
+
+
 # config.json "architecture" -> builder of a layer-list config
-SEQ_ARCHITECTURES = {"Puguzen": puguzen_config, "Naburax": naburax_config, "Fepopel": fepopel_config}
+SEQ_ARCHITECTURES = {"Puguzen": puguzen_config, "Naburax": naburax_config, "Fepopel": fepopel_config,
+                     "Zopupel": zopupel_config}
 
 
 def safetensors_shapes(path: str) -> dict:

@@ -1017,12 +1017,19 @@ SwCols sw_cols(const sd_seq_layer& l) {
     c.dkv = at; at += l.kv_rank + l.rot_dim;
     c.g = at;   at += l.head_gate ? l.heads : 0;
   } else {
-    c.q = at; at += l.heads * l.dim;
-    c.k = at; at += l.kv_heads * l.dim;
-    c.v = at; at += l.kv_heads * l.vdim;
+    const int maps = l.maps > 1 ? l.maps : 1;
+    c.q = at; at += l.heads * maps * l.dim;
+    c.k = at; at += l.kv_shared ? 0 : l.kv_heads * maps * l.dim;
+    c.v = at; at += l.kv_shared || l.value_from_key ? 0 : l.kv_heads * l.vdim;
   }
   c.total = at;
   return c;
+}
+// whether a grouped-query softmax layer needs the general preparation (sd_attn_prep) rather than
+// norms per head alone (sd_qk_head_norm_append)
+inline bool general_prep(const sd_seq_layer& l) {
+  return l.maps > 1 || l.rot_dims > 0 || l.w_in_bias || l.qk_full_norm || l.value_from_key || l.kv_shared ||
+         !l.qk_head_norm;
 }
 inline int act_inputs(int act_kind) { return act_kind == 2 ? 1 : 2; }   // matrices an activation of sd_act_rows reads
 PnCols pn_cols(const sd_seq_layer& l) {
@@ -1061,9 +1068,10 @@ SeqWs plan_seq(const sd_seq_model& m, int rows, int n_out, int max_ctx) {
       up(proj, (size_t)c.total);
       need(l.w_in_tiled, wr, c.total, W);
       need(l.w_o_tiled, wr, W, l.heads * l.vdim);
-      up(hv, (size_t)l.heads * l.vdim);
-      up(attn, sd_masked_softmax_attention_scratch_bytes(rows, l.heads, l.kind == SD_MIX_LATENT ? l.kv_rank : l.vdim,
-                                                         l.window, 0, l.chunk, max_ctx));
+      const int maps = l.kind == SD_MIX_SOFTMAX && l.maps > 1 ? l.maps : 1;
+      up(hv, (size_t)l.heads * maps * l.vdim);
+      up(attn, sd_multimap_softmax_attention_scratch_bytes(rows, l.heads, maps, l.kind == SD_MIX_LATENT ? l.kv_rank : l.vdim,
+                                                           l.window, 0, l.chunk, max_ctx));
       if (l.kind == SD_MIX_LATENT) {
         up(qe, (size_t)l.heads * (l.kv_rank + l.rot_dim));
         up(hv, (size_t)l.heads * l.kv_rank);
@@ -1207,7 +1215,10 @@ extern "C" sd_seq_model* sd_seq_model_create(const sd_seq_model_desc* desc) {
       else if ((l.w_in_tiled || l.w_o_tiled || l.w_ff_in_tiled || l.w_down_tiled || l.w_shared_in_tiled || l.w_shared_down_tiled) && desc->weights_f32) bad = "tiled matrices are bf16";
       else if (l.kind == SD_MIX_LATENT && (l.q_rank != 0 || l.kv_rank < 1 || l.kv_rank > 512 || l.rot_dim < 0 || l.rot_dims < 0 || l.rot_dims > l.rot_dim ||
                l.rot_dims % 2 || (l.rot_dims && !l.inv_freq) || !l.dkv_norm_w || !l.w_uk_t || !l.w_uv)) bad = "latent size / rotary dims / a null latent weight";
-      else if (l.kind == SD_MIX_SOFTMAX && (l.kv_heads < 1 || l.heads % l.kv_heads || l.vdim > 512 || !l.v_cache || !l.qk_head_norm || !l.q_norm_w || !l.k_norm_w)) bad = "attention needs kv heads that divide the heads, vdim <= 512, a value cache and per-head norms";
+      else if (l.kind == SD_MIX_SOFTMAX && (l.kv_heads < 1 || l.heads % l.kv_heads || l.vdim > 512 || !l.v_cache)) bad = "attention needs kv heads that divide the heads, vdim <= 512 and a value cache";
+      else if (l.kind == SD_MIX_SOFTMAX && ((l.qk_head_norm && l.qk_full_norm) || ((l.qk_head_norm || l.qk_full_norm) && (!l.q_norm_w || (!l.kv_shared && !l.k_norm_w))))) bad = "q and k are normed per head or over the whole projection, with weights for both";
+      else if (l.kind == SD_MIX_SOFTMAX && (l.maps < 0 || l.maps > 2 || (l.value_from_key && (l.maps > 1 || l.vdim != l.dim || l.kv_shared)) || (l.kv_shared && i == 0))) bad = "one or two score maps; values taken from keys need one map and vdim == dim; shared keys need an earlier layer";
+      else if (l.kind == SD_MIX_SOFTMAX && (l.rot_dims < 0 || l.rot_dims % 2 || l.rot_dims > l.dim || (l.rot_dims && !l.inv_freq))) bad = "rotary dims";
       else if (l.ff < 0 || (l.ff > 0 && (l.n_experts > 0 || l.ff_act < 0 || l.ff_act > 2 || !(l.w_ff_in || l.w_ff_in_tiled) || !(l.w_down || l.w_down_tiled)))) bad = "a dense feed-forward needs its two matrices and a known activation, and excludes experts";
       else if (l.n_experts > 0 && (l.top < 1 || l.top > l.n_experts || l.expert_ff < 1 || !l.w_router || !l.w_gate_up || !l.w_down_e || l.expert_act < 0 || l.expert_act > 1)) bad = "routed experts need top <= experts, their matrices and a known activation";
       else if (l.shared_ff < 0 || (l.shared_ff > 0 && (l.n_experts < 1 || l.shared_act < 0 || l.shared_act > 2 || !(l.w_shared_in || l.w_shared_in_tiled) || !(l.w_shared_down || l.w_shared_down_tiled)))) bad = "a shared expert stands beside routed experts and needs its matrices";
@@ -1420,22 +1431,41 @@ int sandwich_layer(const sd_seq_model& m, const sd_seq_layer& l, const sd_seq_la
     SQ_TRY(seq_linear(l.w_o, l.w_o_tiled, f32, y, nullptr, (int64_t)H * dv, yb, (int64_t)H * dv, nullptr, mix, W, R, W,
                       H * dv, wide_ws, w.wide_bytes, stream));
   } else {
-    const int G = l.kv_heads;
-    SQ_TRY(sd_qk_head_norm_append(proj + c.q, H, l.q_norm_w, proj + c.k, G, dk, l.k_norm_w, proj + c.v, dv, ld, f32, eps,
-                                  l.k_cache, l.v_cache, b.row_pos, b.row_slot, b.block_tables, b.max_blocks, b.page,
-                                  R, stream));
-    SQ_TRY(sd_masked_softmax_attention(proj + c.q, ld, l.k_cache, l.v_cache, f32, b.row_pos, b.row_slot,
-                                       b.block_tables, b.max_blocks, b.page, R, H, G, dk, dv, l.window, 0, l.chunk,
-                                       l.score_scale, l.softcap, l.sinks, o, l.w_o_tiled ? yb : nullptr,
-                                       base + w.attn, w.attn_bytes, stream));
-    SQ_TRY(seq_linear(l.w_o, l.w_o_tiled, f32, o, nullptr, (int64_t)H * dv, yb, (int64_t)H * dv, nullptr, mix, W, R, W,
-                      H * dv, wide_ws, w.wide_bytes, stream));
+    const int G = l.kv_heads, maps = l.maps > 1 ? l.maps : 1;
+    if (general_prep(l)) {
+      // biases, norms, rotary turn, and the append of keys and values (unless another layer's are read): one launch
+      const char* bias = (const char*)l.w_in_bias;
+      const size_t es = f32 ? sizeof(float) : sizeof(bf16_t);
+      SQ_TRY(sd_attn_prep(proj + c.q, H * maps, l.kv_shared ? nullptr : proj + c.k, G * maps, dk,
+                          l.kv_shared || l.value_from_key ? nullptr : proj + c.v, G, dv, l.value_from_key, ld,
+                          bias ? bias + (size_t)c.q * es : nullptr, bias && !l.kv_shared ? bias + (size_t)c.k * es : nullptr,
+                          l.qk_full_norm ? 1 : (l.qk_head_norm ? 2 : 0), l.q_norm_w, l.k_norm_w, f32, eps, l.rot_dims,
+                          l.rot_layout, l.inv_freq, l.rot_mag != 0.f ? l.rot_mag : 1.f, l.k_cache, l.v_cache, b.row_pos,
+                          b.row_slot, b.block_tables, b.max_blocks, b.page, R, stream));
+    } else {
+      SQ_TRY(sd_qk_head_norm_append(proj + c.q, H, l.q_norm_w, proj + c.k, G, dk, l.k_norm_w, proj + c.v, dv, ld, f32,
+                                    eps, l.k_cache, l.v_cache, b.row_pos, b.row_slot, b.block_tables, b.max_blocks,
+                                    b.page, R, stream));
+    }
+    bf16_t* y_b = l.w_o_tiled ? yb : nullptr;
+    SQ_TRY(sd_multimap_softmax_attention(proj + c.q, ld, l.k_cache, l.v_cache, f32, b.row_pos, b.row_slot,
+                                         b.block_tables, b.max_blocks, b.page, R, H, G, maps, dk, dv, l.window, 0,
+                                         l.chunk, l.score_scale, l.softcap, l.sinks, o, maps > 1 ? nullptr : y_b,
+                                         base + w.attn, w.attn_bytes, stream));
+    const float* heads_out = o;
+    if (maps > 1) {   // the two maps of a head put together, the head's difference normed
+      SQ_TRY(sd_diff_combine_rows(o, l.diff_lambda, eps, l.diff_scale, y, y_b, R, H, dv, rnd, stream));
+      heads_out = y;
+    }
+    SQ_TRY(seq_linear(l.w_o, l.w_o_tiled, f32, heads_out, nullptr, (int64_t)H * dv, yb, (int64_t)H * dv, nullptr, mix, W,
+                      R, W, H * dv, wide_ws, w.wide_bytes, stream));
   }
+  const float mult = l.residual_mult != 0.f ? l.residual_mult : 1.f;
   if (!has_ff)
-    return sd_residual_norm(x, mix, 1, nullptr, nullptr, 0, l.post_norm_w, next_add, next_norm, f32, eps, x_copy, h, hb,
-                            R, W, stream);
-  SQ_TRY(sd_residual_norm(x, mix, 1, nullptr, nullptr, 0, l.post_norm_w, nullptr, l.norm2_w, f32, eps, nullptr, h, hb, R,
-                          W, stream));
+    return sd_residual_norm_scaled(x, mix, 1, l.w_o_bias, nullptr, nullptr, 0, l.post_norm_w, mult, next_add, next_norm,
+                                   f32, eps, x_copy, h, hb, R, W, stream);
+  SQ_TRY(sd_residual_norm_scaled(x, mix, 1, l.w_o_bias, nullptr, nullptr, 0, l.post_norm_w, mult, nullptr, l.norm2_w,
+                                 f32, eps, nullptr, h, hb, R, W, stream));
   if (l.ff > 0) {
     const int F = l.ff, n_in = act_inputs(l.ff_act);
     SQ_TRY(seq_linear(l.w_ff_in, l.w_ff_in_tiled, f32, h, nullptr, W, hb, W, nullptr, proj, (int64_t)n_in * F, R,
@@ -1444,8 +1474,8 @@ int sandwich_layer(const sd_seq_model& m, const sd_seq_layer& l, const sd_seq_la
                        l.w_down_tiled ? actb : nullptr, F, R, F, l.ff_act, rnd, stream));
     SQ_TRY(seq_linear(l.w_down, l.w_down_tiled, f32, proj, nullptr, (int64_t)n_in * F, actb, F, nullptr, ffo, W, R, W,
                       F, wide_ws, w.wide_bytes, stream));
-    return sd_residual_norm(x, ffo, 1, nullptr, nullptr, 0, l.post_norm2_w, next_add, next_norm, f32, eps, x_copy, h,
-                            hb, R, W, stream);
+    return sd_residual_norm_scaled(x, ffo, 1, nullptr, nullptr, nullptr, 0, l.post_norm2_w, mult, next_add, next_norm,
+                                   f32, eps, x_copy, h, hb, R, W, stream);
   }
   float* rlog = (float*)(base + w.rlog);
   int32_t* sel_e = (int32_t*)(base + w.sel_e);
@@ -1453,9 +1483,10 @@ int sandwich_layer(const sd_seq_model& m, const sd_seq_layer& l, const sd_seq_la
   float* dn = (float*)(base + w.dn);
   float* sg = (float*)(base + w.sg);
   const bool gated_shared = l.shared_ff > 0 && l.w_shared_gate;
-  SQ_TRY(sd_moe_route_rows_gated(h, W, l.w_router, f32, rlog, sel_e, sel_w, R, l.n_experts, W, l.top, l.route_score,
-                                 l.route_renorm, l.route_renorm_eps, l.route_scale != 0.f ? l.route_scale : 1.f,
-                                 gated_shared ? l.w_shared_gate : nullptr, gated_shared ? 1 : 0, sg, stream));
+  SQ_TRY(sd_moe_route_rows_biased(h, W, l.w_router, l.router_bias, f32, rlog, sel_e, sel_w, R, l.n_experts, W, l.top,
+                                  l.route_score, l.route_renorm, l.route_renorm_eps,
+                                  l.route_scale != 0.f ? l.route_scale : 1.f, gated_shared ? l.w_shared_gate : nullptr,
+                                  gated_shared ? 1 : 0, sg, stream));
   SQ_TRY(sd_moe_experts(h, hb, W, sel_e, sel_w, l.w_gate_up, l.w_down_e, f32, dn, R, l.top, l.n_experts, l.expert_ff, W,
                         l.expert_scale_input, l.expert_act, base + w.moe, w.moe_bytes, stream));
   if (l.shared_ff > 0) {
@@ -1467,8 +1498,8 @@ int sandwich_layer(const sd_seq_model& m, const sd_seq_layer& l, const sd_seq_la
     SQ_TRY(seq_linear(l.w_shared_down, l.w_shared_down_tiled, f32, proj, nullptr, (int64_t)n_in * F, actb, F, nullptr,
                       ffo, W, R, W, F, wide_ws, w.wide_bytes, stream));
   }
-  return sd_residual_norm(x, dn, l.top, l.shared_ff > 0 ? ffo : nullptr, gated_shared ? sg : nullptr, 1,
-                          l.post_norm2_w, next_add, next_norm, f32, eps, x_copy, h, hb, R, W, stream);
+  return sd_residual_norm_scaled(x, dn, l.top, nullptr, l.shared_ff > 0 ? ffo : nullptr, gated_shared ? sg : nullptr, 1,
+                                 l.post_norm2_w, mult, next_add, next_norm, f32, eps, x_copy, h, hb, R, W, stream);
 }
 }  // namespace
 

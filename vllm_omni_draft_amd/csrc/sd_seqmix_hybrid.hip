@@ -198,6 +198,9 @@ __device__ __forceinline__ void score_key(const KT_* __restrict__ kr, const floa
 // n_splits > 1 (few rows): workgroup (.., .., z) takes tile z / n_hgroups of the row's keys only
 // and leaves its maximum, its sum of weights and its unnormalised weighted values in part_ml /
 // part_acc; softmax_merge_kernel puts a row's tiles together in tile order.
+// maps > 1: a head holds `maps` queries of dk channels (unit h * maps + m of a row of q), the key
+// cache `maps` key rows per kv head (cache head g * maps + m), and every map reads the kv head's
+// one value row; blockIdx.y counts key heads, and out / sinks count units.
 template <typename T, int NH, int NC, int KT>
 __global__ __launch_bounds__(256) void window_softmax_attn_kernel(
     const float* __restrict__ q, int64_t ldq, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
@@ -205,7 +208,7 @@ __global__ __launch_bounds__(256) void window_softmax_attn_kernel(
     const int32_t* __restrict__ block_tables, int max_blocks, int page, int H, int G, int dk, int dv, int window,
     int keep_first, float scale, float* __restrict__ out, bf16_t* __restrict__ out_b, int n_hgroups, int n_splits,
     float* __restrict__ part_acc, float* __restrict__ part_ml, int chunk, float softcap,
-    const float* __restrict__ sinks) {
+    const float* __restrict__ sinks, int maps) {
   extern __shared__ float lds[];
   constexpr int nthr = 256, nw = 4, PARTS = nthr / KT, KW = KT / 64;
   unsigned long long* vat = reinterpret_cast<unsigned long long*>(lds);  // [KT] cache row of the key
@@ -216,19 +219,21 @@ __global__ __launch_bounds__(256) void window_softmax_attn_kernel(
   float* corr = l_run + NH;                                              // [NH]
   float* red = corr + NH;                                                // [nw][dv]
   float* ps = red + nw * dv;                                             // [PARTS][NH][KT] (PARTS > 1)
-  const int r = blockIdx.x, g = blockIdx.y, tid = threadIdx.x;
+  const int r = blockIdx.x, gk = blockIdx.y, g = gk / maps, mp = gk % maps, tid = threadIdx.x;
   const int hgroup = blockIdx.z % n_hgroups, split = blockIdx.z / n_hgroups;
-  const int qh = H / G;
-  const int h0 = g * qh + hgroup * NH;
+  const int qh = H / G, HM = H * maps, GM = G * maps;
+  const int hh0 = g * qh + hgroup * NH;            // the group's first query head
+  const int h0 = hh0 * maps + mp;                  // ... and its unit; the next head's is `maps` further
   const int nh = qh - hgroup * NH < NH ? qh - hgroup * NH : NH;
   const int i = row_pos[r];
   const int32_t* tbl = block_tables + (size_t)row_slot[r] * max_blocks;
-  for (int c = tid; c < nh * dk; c += nthr) qs[c] = q[(size_t)r * ldq + (size_t)h0 * dk + c];
+  for (int c = tid; c < nh * dk; c += nthr)
+    qs[c] = q[(size_t)r * ldq + (size_t)(h0 + (c / dk) * maps) * dk + c % dk];
   if (tid < NH) {
     // (a sink is one more term exp(sink) of the denominator, with no key and no value: the first
     // tile's workgroup starts its running maximum and sum from it)
     const bool sunk = sinks && split == 0 && tid < nh;
-    m_run[tid] = sunk ? sinks[h0 + tid] : -INFINITY;
+    m_run[tid] = sunk ? sinks[h0 + tid * maps] : -INFINITY;
     l_run[tid] = sunk ? 1.f : 0.f;
   }
   int t_first = i - window + 1 > 0 ? i - window + 1 : 0;
@@ -259,9 +264,9 @@ __global__ __launch_bounds__(256) void window_softmax_attn_kernel(
       for (int hq = 0; hq < NH; ++hq) s[hq] = 0.f;
       if (idx < key_hi) {
         const int j = idx < n_kept ? idx : t_first + (idx - n_kept);
-        const size_t at = ((size_t)tbl[j / page] * G + g) * page + j % page;
+        const size_t at = ((size_t)tbl[j / page] * GM + gk) * page + j % page;
         if (c_hi > c_lo) score_key<T, NH>(k_cache + at * dk + c_lo, qs + c_lo, dk, c_hi - c_lo, nh, vec, s);
-        if (part == 0) vat[key] = at;
+        if (part == 0) vat[key] = ((size_t)tbl[j / page] * G + g) * page + j % page;
       }
       if constexpr (PARTS == 1) {
 #pragma unroll
@@ -365,15 +370,15 @@ __global__ __launch_bounds__(256) void window_softmax_attn_kernel(
         for (int u = 1; u < nw; ++u) o += red[u * dv + c];
         o *= inv;
         if (n_splits > 1) {
-          part_acc[(((size_t)split * R + r) * H + h0 + hq) * dv + c] = o;
+          part_acc[(((size_t)split * R + r) * HM + h0 + hq * maps) * dv + c] = o;
         } else {
-          const size_t at = (size_t)r * H * dv + (size_t)(h0 + hq) * dv + c;
+          const size_t at = (size_t)r * HM * dv + (size_t)(h0 + hq * maps) * dv + c;
           out[at] = o;
           if (out_b) out_b[at] = (bf16_t)o;
         }
       }
       if (n_splits > 1 && tid == 0) {
-        float* ml = part_ml + (((size_t)split * R + r) * H + h0 + hq) * 2;
+        float* ml = part_ml + (((size_t)split * R + r) * HM + h0 + hq * maps) * 2;
         ml[0] = m_run[hq];
         ml[1] = l_run[hq];
       }
@@ -437,12 +442,13 @@ void launch_softmax_nc(dim3 grid, int kt, size_t lds, hipStream_t st, int nc, co
                        const void* kc, const void* vc, int v_row, const int32_t* row_pos, const int32_t* row_slot,
                        const int32_t* bt, int max_blocks, int page, int H, int G, int dk, int dv, int window,
                        int keep_first, float scale, float* out, bf16_t* out_b, int n_hgroups, int n_splits,
-                       float* part_acc, float* part_ml, int chunk, float softcap, const float* sinks) {
+                       float* part_acc, float* part_ml, int chunk, float softcap, const float* sinks, int maps) {
 #define SD_GO2(NC, KT)                                                                                               \
   window_softmax_attn_kernel<T, NH, NC, KT><<<grid, 256, lds, st>>>(q, ldq, (const T*)kc, (const T*)vc, v_row, row_pos, \
                                                                     row_slot, bt, max_blocks, page, H, G, dk, dv,       \
                                                                     window, keep_first, scale, out, out_b, n_hgroups,   \
-                                                                    n_splits, part_acc, part_ml, chunk, softcap, sinks)
+                                                                    n_splits, part_acc, part_ml, chunk, softcap, sinks, \
+                                                                    maps)
 #define SD_GO(NC)                                          \
   do {                                                     \
     if constexpr (NH <= 4) {                               \
@@ -586,6 +592,110 @@ __global__ __launch_bounds__(256) void qk_head_norm_append_kernel(
 }
 
 // y[r, h, :] *= sigmoid(z[r, h]): one gate per (row, head).  y_b (or nullptr): the result as bf16.
+// Grouped-query attention's preparation in general, per row.  Workgroup (r, 0): the query row of
+// nq units of dk channels in place: + bias, norm (1: over the whole row, weight [nq*dk]; 2: per
+// unit, one weight [dk]), rotary turn of every unit's first `dims` channels.  Workgroup (r, 1): the
+// key row of nk units the same way, then appended (cache head = unit); the value row (G heads of
+// dv channels) appended as it is, or, v_from_k, the key row as it stood after its bias and before
+// norm and turn (then G * dv == nk * dk).  k == nullptr: the layer reads keys and values another
+// layer appended, and only the query is prepared.
+template <typename T>
+__device__ __forceinline__ void prep_units(float* __restrict__ x, int n_units, int dk, const T* __restrict__ bias,
+                                           int norm_kind, const T* __restrict__ w, float eps, int dims, int layout,
+                                           const double* __restrict__ inv_freq, float mag, int pos, float* red,
+                                           T* __restrict__ raw_dst_base, int raw_dv, size_t raw_head_stride) {
+  const int n = n_units * dk;
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < n; c += blockDim.x) {
+    float v = x[c];
+    if (bias) {
+      v += ld_f(bias + c);
+      x[c] = v;
+    }
+    if (raw_dst_base) st_f(raw_dst_base + (size_t)(c / raw_dv) * raw_head_stride + c % raw_dv, v);
+    ss = fmaf(v, v, ss);
+  }
+  if (norm_kind == 1) {
+    ss = block_sum(ss, red);
+    const float rstd = 1.f / sqrtf(ss / (float)n + eps);
+    for (int c = threadIdx.x; c < n; c += blockDim.x) x[c] = x[c] * rstd * ld_f(w + c);
+  }
+  __syncthreads();
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, nw = blockDim.x >> 6;
+  for (int u = wave; u < n_units; u += nw) {     // a wave per unit
+    float* xu = x + (size_t)u * dk;
+    if (norm_kind == 2) {
+      float s2 = 0.f;
+      for (int c = lane; c < dk; c += 64) s2 = fmaf(xu[c], xu[c], s2);
+      s2 = wave_sum(s2);
+      const float rstd = 1.f / sqrtf(s2 / (float)dk + eps);
+      for (int c = lane; c < dk; c += 64) xu[c] = xu[c] * rstd * ld_f(w + c);
+    }
+    for (int i = lane; i < dims / 2; i += 64) {
+      const double a = (double)pos * inv_freq[i];
+      const float cs = (float)cos(a) * mag, sn = (float)sin(a) * mag;
+      const int iu = layout ? 2 * i : i, iv = layout ? 2 * i + 1 : i + dims / 2;
+      const float p = xu[iu], q = xu[iv];
+      xu[iu] = p * cs - q * sn;
+      xu[iv] = q * cs + p * sn;
+    }
+  }
+}
+template <typename T>
+__global__ __launch_bounds__(256) void attn_prep_kernel(
+    float* __restrict__ q, int nq, float* __restrict__ k, int nk, int dk, const float* __restrict__ v, int G, int dv,
+    int v_from_k, int64_t ld, const T* __restrict__ q_bias, const T* __restrict__ k_bias, int norm_kind,
+    const T* __restrict__ q_w, const T* __restrict__ k_w, float eps, int dims, int layout,
+    const double* __restrict__ inv_freq, float mag, const int32_t* __restrict__ row_pos,
+    const int32_t* __restrict__ row_slot, const int32_t* __restrict__ block_tables, int max_blocks, int page,
+    T* __restrict__ k_cache, T* __restrict__ v_cache) {
+  __shared__ float red[4];
+  const int r = blockIdx.x;
+  const int pos = row_pos[r];
+  if (blockIdx.y == 0) {
+    prep_units<T>(q + (size_t)r * ld, nq, dk, q_bias, norm_kind, q_w, eps, dims, layout, inv_freq, mag, pos, red,
+                  nullptr, 1, 0);
+    return;
+  }
+  const int pg = block_tables[(size_t)row_slot[r] * max_blocks + pos / page];
+  float* kr = k + (size_t)r * ld;
+  // (cache rows of one token: head g at ((pg * heads + g) * page + pos % page) * channels)
+  T* v_dst = v_cache + ((size_t)pg * G * page + pos % page) * dv;
+  prep_units<T>(kr, nk, dk, k_bias, norm_kind, k_w, eps, dims, layout, inv_freq, mag, pos, red,
+                v_from_k ? v_dst : nullptr, dv, (size_t)page * dv);
+  __syncthreads();
+  for (int c = threadIdx.x; c < nk * dk; c += blockDim.x)
+    st_f(k_cache + (((size_t)pg * nk + c / dk) * page + pos % page) * dk + c % dk, kr[c]);
+  if (!v_from_k) {
+    const float* vr = v + (size_t)r * ld;
+    for (int c = threadIdx.x; c < G * dv; c += blockDim.x) st_f(v_dst + (size_t)(c / dv) * page * dv + c % dv, vr[c]);
+  }
+}
+
+// Two score maps per head put together: t = a[r, h, 0] - lambda * a[r, h, 1], then t divided by its
+// root mean square over the head's dv channels and multiplied by out_scale.  A wave per (row, head).
+__global__ __launch_bounds__(256) void diff_combine_kernel(const float* __restrict__ a, float lambda, float eps,
+                                                           float out_scale, float* __restrict__ y,
+                                                           bf16_t* __restrict__ y_b, int n_pairs, int dv, int round) {
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int p = blockIdx.x * (blockDim.x >> 6) + wave;     // (row, head)
+  if (p >= n_pairs) return;
+  const float* a1 = a + (size_t)p * 2 * dv;
+  const float* a2 = a1 + dv;
+  float ss = 0.f;
+  for (int c = lane; c < dv; c += 64) {
+    const float t = a1[c] - lambda * a2[c];
+    ss = fmaf(t, t, ss);
+  }
+  ss = wave_sum(ss);
+  const float f = out_scale / sqrtf(ss / (float)dv + eps);
+  for (int c = lane; c < dv; c += 64) {
+    const float o = maybe_round((a1[c] - lambda * a2[c]) * f, round);
+    y[(size_t)p * dv + c] = o;
+    if (y_b) y_b[(size_t)p * dv + c] = (bf16_t)o;
+  }
+}
+
 __global__ void head_gate_kernel(float* __restrict__ y, int64_t ldy, const float* __restrict__ z, int64_t ldz,
                                  bf16_t* __restrict__ y_b, int64_t ldyb, int H, int dv, int round) {
   const int r = blockIdx.x;
@@ -851,7 +961,8 @@ __global__ __launch_bounds__(1024) void moe_route_rows_kernel(const float* __res
                                                              int E, int K, int top, int score_kind, int renorm,
                                                              int round, float renorm_eps, float weight_scale,
                                                              const T* __restrict__ w_gate, int n_gate,
-                                                             float* __restrict__ gate_out) {
+                                                             float* __restrict__ gate_out,
+                                                             const float* __restrict__ bias) {
   extern __shared__ float sc[];   // [E]
   const int r = blockIdx.x, wave = threadIdx.x >> 6, lane = threadIdx.x & 63, nw = blockDim.x >> 6;
   const float* xr = x + (size_t)r * ldx;
@@ -875,6 +986,7 @@ __global__ __launch_bounds__(1024) void moe_route_rows_kernel(const float* __res
     acc = wave_sum(acc);
     if (lane == 0) {
       if (e < E) {
+        if (bias) acc += bias[e];
         sc[e] = acc;
         if (logits) logits[(size_t)r * E + e] = acc;
       } else {
@@ -1451,7 +1563,7 @@ __global__ __launch_bounds__(256) void residual_norm_kernel(
     float* __restrict__ x, const float* __restrict__ a, int n_a, const float* __restrict__ b,
     const float* __restrict__ b_gate, int64_t ldg, const T* __restrict__ w_post, const T* __restrict__ add,
     const T* __restrict__ w_next, float eps, float* __restrict__ x_copy, float* __restrict__ h,
-    bf16_t* __restrict__ h_b, int W, int round) {
+    bf16_t* __restrict__ h_b, int W, int round, const T* __restrict__ a_bias, float mult) {
   extern __shared__ float row[];   // [W]
   __shared__ float red[4];
   const int r = blockIdx.x;
@@ -1463,6 +1575,7 @@ __global__ __launch_bounds__(256) void residual_norm_kernel(
       float v = a[((size_t)r * n_a) * W + c];
       for (int j = 1; j < n_a; ++j) v += a[((size_t)r * n_a + j) * W + c];
       if (b) v += gate * b[(size_t)r * W + c];
+      if (a_bias) v += ld_f(a_bias + c);
       row[c] = v;
       ss = fmaf(v, v, ss);
     }
@@ -1472,7 +1585,7 @@ __global__ __launch_bounds__(256) void residual_norm_kernel(
   float ss2 = 0.f;
   for (int c = threadIdx.x; c < W; c += blockDim.x) {
     float xn = x[(size_t)r * W + c];
-    if (a) xn += row[c] * rstd * ld_f(w_post + c);
+    if (a) xn += mult * (row[c] * rstd * ld_f(w_post + c));
     if (x_copy) x_copy[(size_t)r * W + c] = xn;
     if (add) xn += ld_f(add + c);
     if (a || add) x[(size_t)r * W + c] = xn;
@@ -1517,7 +1630,7 @@ __global__ __launch_bounds__(1024) void residual_norm_quad_kernel(
     float* __restrict__ x, const float* __restrict__ a, int n_a, const float* __restrict__ b,
     const float* __restrict__ b_gate, int64_t ldg, const T* __restrict__ w_post, const T* __restrict__ add,
     const T* __restrict__ w_next, float eps, float* __restrict__ x_copy, float* __restrict__ h,
-    bf16_t* __restrict__ h_b, int W, int round) {
+    bf16_t* __restrict__ h_b, int W, int round, const T* __restrict__ a_bias, float mult) {
   extern __shared__ float row[];   // [W]
   __shared__ float red[16];
   const int r = blockIdx.x, nq = W / 4;
@@ -1529,6 +1642,7 @@ __global__ __launch_bounds__(1024) void residual_norm_quad_kernel(
       f32x4 v = Quad<float>::ld(a + ((size_t)r * n_a) * W + 4 * c);
       for (int j = 1; j < n_a; ++j) v += Quad<float>::ld(a + ((size_t)r * n_a + j) * W + 4 * c);
       if (b) v += gate * Quad<float>::ld(b + (size_t)r * W + 4 * c);
+      if (a_bias) v += Quad<T>::ld(a_bias + 4 * c);
       *reinterpret_cast<f32x4*>(row + 4 * c) = v;
 #pragma unroll
       for (int i = 0; i < 4; ++i) ss = fmaf(v[i], v[i], ss);
@@ -1542,7 +1656,7 @@ __global__ __launch_bounds__(1024) void residual_norm_quad_kernel(
     if (a) {
       const f32x4 t = *reinterpret_cast<const f32x4*>(row + 4 * c), wp = Quad<T>::ld(w_post + 4 * c);
 #pragma unroll
-      for (int i = 0; i < 4; ++i) xn[i] += t[i] * rstd * wp[i];
+      for (int i = 0; i < 4; ++i) xn[i] += mult * (t[i] * rstd * wp[i]);
     }
     if (x_copy) *reinterpret_cast<f32x4*>(x_copy + (size_t)r * W + 4 * c) = xn;
     if (add) xn += Quad<T>::ld(add + 4 * c);
@@ -1704,6 +1818,55 @@ extern "C" int sd_qk_head_norm_append(float* q, int H, const void* q_norm_w, flo
   return SD_OK;
 }
 
+extern "C" int sd_attn_prep(float* q, int n_q_units, float* k, int n_k_units, int dk, const float* v, int G, int dv,
+                            int value_from_key, int64_t ld, const void* q_bias, const void* k_bias, int norm_kind,
+                            const void* q_norm_w, const void* k_norm_w, int w_f32, float eps, int rot_dims,
+                            int rot_layout, const double* inv_freq, float mag, void* k_cache, void* v_cache,
+                            const int32_t* row_pos, const int32_t* row_slot, const int32_t* block_tables,
+                            int max_blocks, int page, int n_rows, sd_stream_t stream) {
+  SD_REQUIRE(q && row_pos && n_rows >= 1 && n_q_units >= 1 && dk >= 1 && ld >= (int64_t)n_q_units * dk, SD_ERR_INVALID,
+             "sd_attn_prep: bad argument");
+  SD_REQUIRE(norm_kind >= 0 && norm_kind <= 2 && (norm_kind == 0 || (q_norm_w && (!k || k_norm_w))), SD_ERR_INVALID,
+             "sd_attn_prep: norm kind %d unknown, or a norm without its weights", norm_kind);
+  SD_REQUIRE(rot_dims >= 0 && rot_dims % 2 == 0 && rot_dims <= dk && (rot_dims == 0 || inv_freq), SD_ERR_INVALID,
+             "sd_attn_prep: rotary dims %d (dim %d)", rot_dims, dk);
+  if (k) {
+    SD_REQUIRE(n_k_units >= 1 && G >= 1 && dv >= 1 && k_cache && v_cache && row_slot && block_tables && page >= 1 &&
+                   max_blocks >= 1 && ld >= (int64_t)n_k_units * dk,
+               SD_ERR_INVALID, "sd_attn_prep: keys without their caches or page table");
+    SD_REQUIRE(value_from_key ? (int64_t)G * dv == (int64_t)n_k_units * dk : (v != nullptr && ld >= (int64_t)G * dv),
+               SD_ERR_INVALID, "sd_attn_prep: values missing, or values taken from keys of another size");
+  }
+  hipStream_t st = (hipStream_t)stream;
+  const dim3 grid(n_rows, k ? 2 : 1);
+  if (w_f32)
+    attn_prep_kernel<float><<<grid, 256, 0, st>>>(q, n_q_units, k, n_k_units, dk, v, G, dv, value_from_key, ld,
+                                                  (const float*)q_bias, (const float*)k_bias, norm_kind,
+                                                  (const float*)q_norm_w, (const float*)k_norm_w, eps, rot_dims,
+                                                  rot_layout, inv_freq, mag, row_pos, row_slot, block_tables,
+                                                  max_blocks, page, (float*)k_cache, (float*)v_cache);
+  else
+    attn_prep_kernel<bf16_t><<<grid, 256, 0, st>>>(q, n_q_units, k, n_k_units, dk, v, G, dv, value_from_key, ld,
+                                                   (const bf16_t*)q_bias, (const bf16_t*)k_bias, norm_kind,
+                                                   (const bf16_t*)q_norm_w, (const bf16_t*)k_norm_w, eps, rot_dims,
+                                                   rot_layout, inv_freq, mag, row_pos, row_slot, block_tables,
+                                                   max_blocks, page, (bf16_t*)k_cache, (bf16_t*)v_cache);
+  SD_CHECK_LAUNCH("sd_attn_prep");
+  return SD_OK;
+}
+
+extern "C" int sd_diff_combine_rows(const float* a, float lambda, float eps, float out_scale, float* y, void* y_bf16,
+                                    int n_rows, int H, int dv, int round_bf16_out, sd_stream_t stream) {
+  SD_REQUIRE(a && y && n_rows >= 1 && H >= 1 && dv >= 1, SD_ERR_INVALID, "sd_diff_combine_rows: bad argument");
+  const long long pairs = (long long)n_rows * H;
+  SD_REQUIRE(pairs <= 0x7fffffff, SD_ERR_UNSUPPORTED, "sd_diff_combine_rows: too many (row, head) pairs");
+  diff_combine_kernel<<<(unsigned)((pairs + 3) / 4), 256, 0, (hipStream_t)stream>>>(a, lambda, eps, out_scale, y,
+                                                                                   (bf16_t*)y_bf16, (int)pairs, dv,
+                                                                                   round_bf16_out);
+  SD_CHECK_LAUNCH("sd_diff_combine_rows");
+  return SD_OK;
+}
+
 extern "C" int sd_head_gate_rows(float* y, int64_t ldy, const float* z, int64_t ldz, void* y_bf16, int64_t ldyb,
                                  int n_rows, int H, int dv, int round_bf16_out, sd_stream_t stream) {
   SD_REQUIRE(y && z && n_rows >= 1 && H >= 1 && dv >= 1 && ldy >= (int64_t)H * dv && ldz >= H, SD_ERR_INVALID,
@@ -1750,7 +1913,13 @@ extern "C" int sd_cache_append(const float* k, int64_t ldk, const float* v, int6
 
 extern "C" size_t sd_masked_softmax_attention_scratch_bytes(int n_rows, int H, int dv, int window, int keep_first,
                                                              int chunk, int max_ctx) {
-  if (n_rows < 1 || n_rows > kSplitRows || H < 1 || dv < 1 || window < 1) return 0;
+  return sd_multimap_softmax_attention_scratch_bytes(n_rows, H, 1, dv, window, keep_first, chunk, max_ctx);
+}
+
+extern "C" size_t sd_multimap_softmax_attention_scratch_bytes(int n_rows, int H, int maps, int dv, int window,
+                                                               int keep_first, int chunk, int max_ctx) {
+  if (n_rows < 1 || n_rows > kSplitRows || H < 1 || maps < 1 || dv < 1 || window < 1) return 0;
+  H *= maps;
   long long max_keys = (long long)(chunk > 0 && chunk < window ? chunk : window) + (keep_first > 0 ? keep_first : 0);
   if (max_keys > max_ctx) max_keys = max_ctx;
   const int splits = (int)((max_keys + kSplitKeys - 1) / kSplitKeys);
@@ -1763,18 +1932,32 @@ extern "C" int sd_masked_softmax_attention(const float* q, int64_t ldq, const vo
                                            int G, int dk, int dv, int window, int keep_first, int chunk, float scale,
                                            float softcap, const float* sinks, float* out, void* out_bf16,
                                            void* scratch, size_t scratch_bytes, sd_stream_t stream) {
+  return sd_multimap_softmax_attention(q, ldq, k_cache, v_cache, cache_f32, row_pos, row_slot, block_tables, max_blocks,
+                                       page, n_rows, H, G, 1, dk, dv, window, keep_first, chunk, scale, softcap, sinks,
+                                       out, out_bf16, scratch, scratch_bytes, stream);
+}
+
+extern "C" int sd_multimap_softmax_attention(const float* q, int64_t ldq, const void* k_cache, const void* v_cache,
+                                             int cache_f32, const int32_t* row_pos, const int32_t* row_slot,
+                                             const int32_t* block_tables, int max_blocks, int page, int n_rows, int H,
+                                             int G, int maps, int dk, int dv, int window, int keep_first, int chunk,
+                                             float scale, float softcap, const float* sinks, float* out,
+                                             void* out_bf16, void* scratch, size_t scratch_bytes, sd_stream_t stream) {
   SD_REQUIRE(q && k_cache && row_pos && row_slot && block_tables && out, SD_ERR_INVALID,
              "sd_masked_softmax_attention: null argument");
   SD_REQUIRE(n_rows >= 1 && H >= 1 && G >= 1 && H % G == 0 && dk >= 1 && window >= 1 && keep_first >= 0 && page >= 1 &&
-                 chunk >= 0 && softcap >= 0.f,
+                 chunk >= 0 && softcap >= 0.f && maps >= 1 && (maps == 1 || v_cache) &&
+                 ldq >= (int64_t)H * maps * dk,
              SD_ERR_INVALID, "sd_masked_softmax_attention: bad shape");
   SD_REQUIRE(dv >= 1 && dv <= 512 && (v_cache || dv <= dk), SD_ERR_UNSUPPORTED,
              "sd_masked_softmax_attention: value size %d outside 1..512 (or above the key row it is part of)", dv);
   hipStream_t st = (hipStream_t)stream;
   const int qh = H / G;
-  const size_t need = sd_masked_softmax_attention_scratch_bytes(n_rows, H, dv, window, keep_first, chunk, max_blocks * page);
+  const int HM = H * maps;
+  const size_t need = sd_multimap_softmax_attention_scratch_bytes(n_rows, H, maps, dv, window, keep_first, chunk,
+                                                                  max_blocks * page);
   const bool split = need > 0 && scratch && scratch_bytes >= need && sd_aligned16(scratch);
-  const int n_splits = split ? (int)(need / ((size_t)n_rows * H * (dv + 2) * sizeof(float))) : 1;
+  const int n_splits = split ? (int)(need / ((size_t)n_rows * HM * (dv + 2) * sizeof(float))) : 1;
   const int kt = split ? kSplitKeys : 256;   // keys per tile
   // (a cut launch has many workgroups already: fewer heads each, so that a thread scores its key sooner)
   const int cap = split ? 4 : 8;
@@ -1789,12 +1972,12 @@ extern "C" int sd_masked_softmax_attention(const float* q, int64_t ldq, const vo
   const void* vc = v_cache ? v_cache : k_cache;
   const int v_row = v_cache ? dv : dk;
   float* part_acc = split ? (float*)scratch : nullptr;
-  float* part_ml = split ? part_acc + (size_t)n_splits * n_rows * H * dv : nullptr;
-  dim3 grid(n_rows, G, n_hgroups * n_splits);
+  float* part_ml = split ? part_acc + (size_t)n_splits * n_rows * HM * dv : nullptr;
+  dim3 grid(n_rows, G * maps, n_hgroups * n_splits);
 #define SD_NH(T, N)                                                                                                  \
   launch_softmax_nc<T, N>(grid, kt, lds, st, nc, q, ldq, k_cache, vc, v_row, row_pos, row_slot, block_tables,      \
                           max_blocks, page, H, G, dk, dv, window, keep_first, scale, out, (bf16_t*)out_bf16, n_hgroups, \
-                          n_splits, part_acc, part_ml, chunk, softcap, sinks)
+                          n_splits, part_acc, part_ml, chunk, softcap, sinks, maps)
 #define SD_T(T)                      \
   do {                               \
     if (NH == 1) SD_NH(T, 1);        \
@@ -1808,8 +1991,8 @@ extern "C" int sd_masked_softmax_attention(const float* q, int64_t ldq, const vo
 #undef SD_NH
   SD_CHECK_LAUNCH("sd_masked_softmax_attention");
   if (split) {
-    softmax_merge_kernel<<<dim3(n_rows, H), dv <= 64 ? 64 : (dv <= 128 ? 128 : 256), sizeof(float) * n_splits, st>>>(
-        part_acc, part_ml, n_splits, out, (bf16_t*)out_bf16, H, dv);
+    softmax_merge_kernel<<<dim3(n_rows, HM), dv <= 64 ? 64 : (dv <= 128 ? 128 : 256), sizeof(float) * n_splits, st>>>(
+        part_acc, part_ml, n_splits, out, (bf16_t*)out_bf16, HM, dv);
     SD_CHECK_LAUNCH("sd_masked_softmax_attention (merge)");
   }
   return SD_OK;
@@ -1916,6 +2099,15 @@ extern "C" int sd_moe_route_rows_gated(const float* x, int64_t ldx, const void* 
                                        int32_t* sel_expert, float* sel_weight, int n_rows, int E, int K, int top,
                                        int score_kind, int renorm, float renorm_eps, float weight_scale,
                                        const void* w_gate, int n_gate, float* gate_out, sd_stream_t stream) {
+  return sd_moe_route_rows_biased(x, ldx, w_router, nullptr, w_f32, logits, sel_expert, sel_weight, n_rows, E, K, top,
+                                  score_kind, renorm, renorm_eps, weight_scale, w_gate, n_gate, gate_out, stream);
+}
+
+extern "C" int sd_moe_route_rows_biased(const float* x, int64_t ldx, const void* w_router, const float* router_bias,
+                                        int w_f32, float* logits, int32_t* sel_expert, float* sel_weight, int n_rows,
+                                        int E, int K, int top, int score_kind, int renorm, float renorm_eps,
+                                        float weight_scale, const void* w_gate, int n_gate, float* gate_out,
+                                        sd_stream_t stream) {
   SD_REQUIRE(x && w_router && sel_expert && sel_weight && n_rows >= 1 && E >= 1 && K >= 1 && top >= 1 && top <= E &&
                  ldx >= K,
              SD_ERR_INVALID, "sd_moe_route_rows: bad argument (E=%d top=%d)", E, top);
@@ -1927,11 +2119,11 @@ extern "C" int sd_moe_route_rows_gated(const float* x, int64_t ldx, const void* 
   if (w_f32)
     moe_route_rows_kernel<float><<<n_rows, nthr, sizeof(float) * E, st>>>(
         x, ldx, (const float*)w_router, logits, sel_expert, sel_weight, E, K, top, score_kind, renorm, 0, renorm_eps,
-        weight_scale, (const float*)w_gate, n_gate, gate_out);
+        weight_scale, (const float*)w_gate, n_gate, gate_out, router_bias);
   else
     moe_route_rows_kernel<bf16_t><<<n_rows, nthr, sizeof(float) * E, st>>>(
         x, ldx, (const bf16_t*)w_router, logits, sel_expert, sel_weight, E, K, top, score_kind, renorm, 1, renorm_eps,
-        weight_scale, (const bf16_t*)w_gate, n_gate, gate_out);
+        weight_scale, (const bf16_t*)w_gate, n_gate, gate_out, router_bias);
   SD_CHECK_LAUNCH("sd_moe_route_rows");
   return SD_OK;
 }
@@ -2044,6 +2236,15 @@ extern "C" int sd_postnorm_residual(float* x, const float* a, int n_a, float sa,
 extern "C" int sd_residual_norm(float* x, const float* a, int n_a, const float* b, const float* b_gate, int64_t ldg,
                                 const void* w_post, const void* add, const void* w_next, int w_f32, float eps,
                                 float* x_copy, float* h, void* h_bf16, int n_rows, int W, sd_stream_t stream) {
+  return sd_residual_norm_scaled(x, a, n_a, nullptr, b, b_gate, ldg, w_post, 1.f, add, w_next, w_f32, eps, x_copy, h,
+                                 h_bf16, n_rows, W, stream);
+}
+
+extern "C" int sd_residual_norm_scaled(float* x, const float* a, int n_a, const void* a_bias, const float* b,
+                                       const float* b_gate, int64_t ldg, const void* w_post, float mult,
+                                       const void* add, const void* w_next, int w_f32, float eps, float* x_copy,
+                                       float* h, void* h_bf16, int n_rows, int W, sd_stream_t stream) {
+  SD_REQUIRE(!a_bias || a, SD_ERR_INVALID, "sd_residual_norm: a bias without the rows it is added to");
   SD_REQUIRE(x && n_rows >= 1 && W >= 1 && (!a || (w_post && n_a >= 1)) && (!b || a) && (!b_gate || (b && ldg >= 1)) &&
                  (!w_next || h || h_bf16),
              SD_ERR_INVALID, "sd_residual_norm: bad argument");
@@ -2054,28 +2255,30 @@ extern "C" int sd_residual_norm(float* x, const float* a, int n_a, const float* 
   // (weights are 4 or 2 bytes an element: four of them are 16 or 8 bytes, and a vector [W] starts aligned to that
   // when its address is a multiple of 16; `add` may be a row of a table, whose rows are W elements apart)
   if (W % 4 == 0 && W >= 256 && al16(x) && al16(a) && al16(b) && al16(w_post) && al16(w_next) && al16(x_copy) &&
-      al16(h) && al16(h_bf16) && (reinterpret_cast<uintptr_t>(add) & 7) == 0 && (!w_f32 || al16(add))) {
+      al16(h) && al16(h_bf16) && (reinterpret_cast<uintptr_t>(add) & 7) == 0 && (!w_f32 || al16(add)) &&
+      al16(a_bias)) {
     int nthr = ((W / 4 + 63) / 64) * 64;
     if (nthr > 1024) nthr = 1024;
     if (w_f32)
       residual_norm_quad_kernel<float><<<n_rows, nthr, lds, st>>>(x, a, n_a, b, b_gate, ldg, (const float*)w_post,
                                                                   (const float*)add, (const float*)w_next, eps, x_copy,
-                                                                  h, (bf16_t*)h_bf16, W, 0);
+                                                                  h, (bf16_t*)h_bf16, W, 0, (const float*)a_bias, mult);
     else
       residual_norm_quad_kernel<bf16_t><<<n_rows, nthr, lds, st>>>(x, a, n_a, b, b_gate, ldg, (const bf16_t*)w_post,
                                                                    (const bf16_t*)add, (const bf16_t*)w_next, eps,
-                                                                   x_copy, h, (bf16_t*)h_bf16, W, 1);
+                                                                   x_copy, h, (bf16_t*)h_bf16, W, 1,
+                                                                   (const bf16_t*)a_bias, mult);
     SD_CHECK_LAUNCH("sd_residual_norm");
     return SD_OK;
   }
   if (w_f32)
     residual_norm_kernel<float><<<n_rows, 256, lds, st>>>(x, a, n_a, b, b_gate, ldg, (const float*)w_post,
                                                           (const float*)add, (const float*)w_next, eps, x_copy, h,
-                                                          (bf16_t*)h_bf16, W, 0);
+                                                          (bf16_t*)h_bf16, W, 0, (const float*)a_bias, mult);
   else
     residual_norm_kernel<bf16_t><<<n_rows, 256, lds, st>>>(x, a, n_a, b, b_gate, ldg, (const bf16_t*)w_post,
                                                            (const bf16_t*)add, (const bf16_t*)w_next, eps, x_copy, h,
-                                                           (bf16_t*)h_bf16, W, 1);
+                                                           (bf16_t*)h_bf16, W, 1, (const bf16_t*)a_bias, mult);
   SD_CHECK_LAUNCH("sd_residual_norm");
   return SD_OK;
 }

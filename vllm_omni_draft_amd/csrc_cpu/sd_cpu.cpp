@@ -1563,6 +1563,31 @@ extern "C" int sd_residual_norm(float*, const float*, int, const float*, const f
                                 const void*, int, float, float*, float*, void*, int, int, sd_stream_t) {
   UNSUPPORTED("sd_residual_norm");
 }
+extern "C" size_t sd_multimap_softmax_attention_scratch_bytes(int, int, int, int, int, int, int, int) { return 0; }
+extern "C" int sd_multimap_softmax_attention(const float*, int64_t, const void*, const void*, int, const int32_t*,
+                                             const int32_t*, const int32_t*, int, int, int, int, int, int, int, int,
+                                             int, int, int, float, float, const float*, float*, void*, void*, size_t,
+                                             sd_stream_t) {
+  UNSUPPORTED("sd_multimap_softmax_attention");
+}
+extern "C" int sd_attn_prep(float*, int, float*, int, int, const float*, int, int, int, int64_t, const void*,
+                            const void*, int, const void*, const void*, int, float, int, int, const double*, float,
+                            void*, void*, const int32_t*, const int32_t*, const int32_t*, int, int, int, sd_stream_t) {
+  UNSUPPORTED("sd_attn_prep");
+}
+extern "C" int sd_diff_combine_rows(const float*, float, float, float, float*, void*, int, int, int, int, sd_stream_t) {
+  UNSUPPORTED("sd_diff_combine_rows");
+}
+extern "C" int sd_moe_route_rows_biased(const float*, int64_t, const void*, const float*, int, float*, int32_t*, float*,
+                                        int, int, int, int, int, int, float, float, const void*, int, float*,
+                                        sd_stream_t) {
+  UNSUPPORTED("sd_moe_route_rows_biased");
+}
+extern "C" int sd_residual_norm_scaled(float*, const float*, int, const void*, const float*, const float*, int64_t,
+                                       const void*, float, const void*, const void*, int, float, float*, float*, void*,
+                                       int, int, sd_stream_t) {
+  UNSUPPORTED("sd_residual_norm_scaled");
+}
 extern "C" int sd_scale_rows(float*, int64_t, float, int, int, sd_stream_t) { UNSUPPORTED("sd_scale_rows"); }
 extern "C" sd_seq_model* sd_seq_model_create(const sd_seq_model_desc*) {
   set_error("sd_seq_model_create: not provided by the CPU build of the library");

@@ -150,7 +150,10 @@ class SeqCache:
     in k only; a state-space recurrence keeps state[layer] [slots, heads, state, vdim] and the
     tail of its convolution's inputs conv[layer] f32 [slots, taps - 1, channels].  The tensors are
     keyed by the layer's place in the order of running (cfg.runs): a layer that runs several
-    times over keeps a cache for every pass."""
+    times over keeps a cache for every pass.  A softmax attention with several score maps per head
+    keeps that many key rows per kv head and token (cache head = kv head * maps + map) and one value
+    row; a layer that reads another layer's keys and values owns no tensors: kv_source names the
+    run whose tensors it reads."""
 
     def __init__(self, cfg, dtype: torch.dtype, max_seqs: int, num_pages: int, max_seq_len: int,
                  device="cuda"):
@@ -168,9 +171,15 @@ class SeqCache:
         self.pk: Dict[int, torch.Tensor] = {}
         self.pv: Dict[int, torch.Tensor] = {}
         self.conv: Dict[int, torch.Tensor] = {}
+        self.kv_source: Dict[int, int] = {}
         self.has_pages = False
+        run_of = {li: i for i, (li, _) in enumerate(cfg.runs)}   # (a layer others read runs once)
         for i, (li, _) in enumerate(cfg.runs):
             m = cfg.layers[li].mixer
+            if m.kv_from >= 0:
+                self.has_pages = True
+                self.kv_source[i] = run_of[m.kv_from]
+                continue
             if m.kind == "latent_attention":
                 # one row per token serves as key and value: the latent, then the shared rotated part
                 self.has_pages = True
@@ -185,7 +194,7 @@ class SeqCache:
                                            device=device)
             elif m.kind == "softmax_attention":
                 self.has_pages = True
-                self.k[i] = torch.zeros(num_pages, m.kv_heads, PAGE, m.dim, dtype=dtype, device=device)
+                self.k[i] = torch.zeros(num_pages, m.kv_heads * m.maps, PAGE, m.dim, dtype=dtype, device=device)
                 self.v[i] = torch.zeros(num_pages, m.kv_heads, PAGE, m.vdim, dtype=dtype, device=device)
             elif m.kind == "attention":
                 self.has_pages = True
@@ -196,6 +205,13 @@ class SeqCache:
                 self.pv[i] = torch.zeros(num_pages, m.kv_heads, ps, m.vdim, dtype=torch.float32, device=device)
             else:
                 self.state[i] = torch.zeros(max_seqs, m.heads, m.dim, m.vdim, dtype=torch.float32, device=device)
+
+    def keys_of(self, run: int):
+        """The key cache run `run` reads: its own, or the one of the run it shares with."""
+        return self.k.get(self.kv_source.get(run, run))
+
+    def values_of(self, run: int):
+        return self.v.get(self.kv_source.get(run, run))
 
     def pages_of(self, slot: int) -> List[int]:
         return self._host_tables[slot]

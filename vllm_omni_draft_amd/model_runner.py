@@ -249,7 +249,11 @@ class SeqModel:
                     w_o=rm(t.w_o), w_o_tiled=tl(t.w_o), kv_rank=m.kv_rank, rot_dim=m.rot_dim,
                     dkv_norm_w=_ptr(t.dkv_norm_w), w_uk_t=_ptr(t.w_uk_t), w_uv=_ptr(t.w_uv),
                     q_norm_w=_ptr(t.q_norm_w), k_norm_w=_ptr(t.k_norm_w),
-                    k_cache=_ptr(cache.k.get(i)), v_cache=_ptr(cache.v.get(i)),
+                    k_cache=_ptr(cache.keys_of(i)), v_cache=_ptr(cache.values_of(i)),
+                    maps=m.maps, diff_lambda=t.diff_lambda, diff_scale=1.0 - m.diff,
+                    qk_full_norm=int(m.qk_full_norm), value_from_key=int(m.value_is_key),
+                    kv_shared=int(m.kv_from >= 0), w_in_bias=_ptr(t.w_in_bias), w_o_bias=_ptr(t.w_o_bias),
+                    router_bias=_ptr(t.router_bias), residual_mult=cfg.residual_mult,
                     w_ff_in=rm(t.w_ff_in), w_ff_in_tiled=tl(t.w_ff_in), w_down=rm(t.w_down),
                     w_down_tiled=tl(t.w_down), ff_act=acts[spec.ff_act],
                     n_experts=ex.experts if ex else 0, top=ex.top if ex else 0, expert_ff=ex.ff if ex else 0,

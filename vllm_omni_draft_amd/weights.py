@@ -362,6 +362,10 @@ class SeqLayerTensors:
     w_shared_in: object = None                 # a shared expert: [shared_ff, width]
     w_shared_down: object = None               # [width, shared_ff]
     w_shared_gate: Optional[torch.Tensor] = None   # [1, width]
+    w_in_bias: Optional[torch.Tensor] = None   # [w_in's rows]: biases of q and k
+    w_o_bias: Optional[torch.Tensor] = None    # [width]
+    router_bias: Optional[torch.Tensor] = None  # f32 [experts]
+    diff_lambda: float = 0.0                   # differential attention: the second map's factor
 
 
 @dataclass
@@ -540,10 +544,32 @@ def _sandwich_layer(cfg, i: int, get, dev, mat) -> SeqLayerTensors:
             i2 = torch.arange(m.rot_dims // 2, dtype=torch.float64)
             lt.inv_freq = dev(torch.tensor(m.rot_base, dtype=torch.float64) ** (-2.0 * i2 / m.rot_dims), torch.float64)
     else:
-        parts = [get(p + "mix.q", (H * dk, W)), get(p + "mix.k", (G * dk, W)), get(p + "mix.v", (G * dv, W))]
+        from .config import rotary_frequencies
+        own, nq, nk = m.kv_from < 0, H * m.maps * dk, G * m.maps * dk
+        parts = [get(p + "mix.q", (nq, W))]
+        if own:
+            parts += [get(p + "mix.k", (nk, W))] + ([] if m.value_is_key else [get(p + "mix.v", (G * dv, W))])
         lt = SeqLayerTensors(norm_w=dev(get(p + "norm1", (W,))), w_in=mat(torch.cat([t.float() for t in parts])),
                              w_o=mat(get(p + "mix.o", (W, H * dv))), r1_bias=None)
-        lt.q_norm_w, lt.k_norm_w = dev(get(p + "mix.q.norm", (dk,))), dev(get(p + "mix.k.norm", (dk,)))
+        if m.qk_head_norm or m.qk_full_norm:
+            n1, n2 = (dk, dk) if m.qk_head_norm else (nq, nk)
+            lt.q_norm_w = dev(get(p + "mix.q.norm", (n1,)))
+            lt.k_norm_w = dev(get(p + "mix.k.norm", (n2,))) if own else None
+        if m.proj_bias:
+            rows = [get(p + "mix.q.b", (nq,))] + ([get(p + "mix.k.b", (nk,))] if own else [])
+            if own and not m.value_is_key:
+                rows.append(torch.zeros(G * dv))
+            lt.w_in_bias = dev(torch.cat([t.float() for t in rows]))
+            lt.w_o_bias = dev(get(p + "mix.o.b", (W,)))
+        if m.unit_sink:
+            lt.sinks = dev(torch.zeros(H * m.maps), torch.float32)
+        if m.maps == 2:
+            # one number per layer, formed in float32 from the four learned vectors
+            lq1, lk1, lq2, lk2 = (get(p + "mix." + n, (dk,)).float() for n in ("lq1", "lk1", "lq2", "lk2"))
+            lt.diff_lambda = float(torch.exp((lq1 * lk1).sum()) - torch.exp((lq2 * lk2).sum()) + torch.tensor(m.diff))
+        if m.rot_dims:
+            f, mag = rotary_frequencies(m.rot_dims, m.rot_base, m.rot_scaling)
+            lt.inv_freq, lt.rot_mag = dev(f, torch.float64), float(mag)
     lt.post_norm_w = dev(get(p + "norm1b", (W,)))
     ex = l.experts
     if l.ff or ex is not None:
@@ -554,6 +580,8 @@ def _sandwich_layer(cfg, i: int, get, dev, mat) -> SeqLayerTensors:
     if ex is not None:
         gated = ex.act == "silu"
         lt.w_router = dev(get(p + "mlp.router", (ex.experts, W)))
+        if ex.router_bias:
+            lt.router_bias = dev(get(p + "mlp.router.b", (ex.experts,)), torch.float32)
         lt.w_gate_up = dev(torch.stack([
             torch.cat([get(p + f"mlp.e{e}.gate", (ex.ff, W)), get(p + f"mlp.e{e}.up", (ex.ff, W))]) if gated
             else get(p + f"mlp.e{e}.up", (ex.ff, W)) for e in range(ex.experts)]))
@@ -677,9 +705,23 @@ def _sandwich_random_state(cfg, rn) -> Dict[str, torch.Tensor]:
             if m.head_gate:
                 st[p + "mix.g"] = rn(H, W, s=W ** -0.5)
         else:
-            st[p + "mix.q"], st[p + "mix.k"] = rn(H * dk, W, s=W ** -0.5), rn(G * dk, W, s=W ** -0.5)
-            st[p + "mix.v"] = rn(G * dv, W, s=W ** -0.5)
-            st[p + "mix.q.norm"], st[p + "mix.k.norm"] = 1 + rn(dk, s=0.1), 1 + rn(dk, s=0.1)
+            own, nq, nk = m.kv_from < 0, H * m.maps * dk, G * m.maps * dk
+            st[p + "mix.q"] = rn(nq, W, s=W ** -0.5)
+            if own:
+                st[p + "mix.k"] = rn(nk, W, s=W ** -0.5)
+                if not m.value_is_key:
+                    st[p + "mix.v"] = rn(G * dv, W, s=W ** -0.5)
+            if m.qk_head_norm or m.qk_full_norm:
+                st[p + "mix.q.norm"] = 1 + rn(dk if m.qk_head_norm else nq, s=0.1)
+                if own:
+                    st[p + "mix.k.norm"] = 1 + rn(dk if m.qk_head_norm else nk, s=0.1)
+            if m.proj_bias:
+                st[p + "mix.q.b"], st[p + "mix.o.b"] = rn(nq, s=0.2), rn(W, s=0.2)
+                if own:
+                    st[p + "mix.k.b"] = rn(nk, s=0.2)
+            if m.maps == 2:
+                for nm in ("lq1", "lk1", "lq2", "lk2"):
+                    st[p + "mix." + nm] = rn(dk, s=0.3)
         st[p + "mix.o"] = rn(W, H * dv, s=(H * dv) ** -0.5)
         if l.ff:
             st[p + "mlp.gate"], st[p + "mlp.up"] = rn(l.ff, W, s=W ** -0.5), rn(l.ff, W, s=W ** -0.5)
@@ -687,6 +729,8 @@ def _sandwich_random_state(cfg, rn) -> Dict[str, torch.Tensor]:
         ex = l.experts
         if ex is not None:
             st[p + "mlp.router"] = rn(ex.experts, W, s=W ** -0.5)
+            if ex.router_bias:
+                st[p + "mlp.router.b"] = rn(ex.experts, s=0.3)
             names = [f"e{e}" for e in range(ex.experts)] + (["shared"] if ex.shared_ff else [])
             for nm in names:
                 F = ex.shared_ff if nm == "shared" else ex.ff
