@@ -1360,6 +1360,90 @@ def residual_norm(x, a=None, w_post=None, n_a=1, b=None, b_gate=None, add=None, 
     return copy, h
 
 
+def multimap_softmax_attention(q, k_cache, v_cache, row_pos, row_slot, block_tables, H, G, maps, dk, dv, scale,
+                               window=0, keep_first=0, chunk=0, softcap=0.0, sinks=None, split=True) -> torch.Tensor:
+    """masked_softmax_attention with `maps` score maps per head: q f32 [rows, H*maps*dk], k_cache
+    [pages, G*maps, PAGE, dk], v_cache [pages, G, PAGE, dv]; returns every map's own output, f32
+    [rows, H*maps*dv].  sinks f32 [H*maps]."""
+    _f32(q, "q")
+    if sinks is not None:
+        _f32(sinks, "sinks")
+    window = int(window) or 0x7fffffff
+    out = torch.empty(q.shape[0], H * maps * dv, dtype=torch.float32, device=q.device)
+    lib = _lib.load()
+    n = int(lib.sd_multimap_softmax_attention_scratch_bytes(q.shape[0], H, maps, dv, window, int(keep_first),
+                                                            int(chunk), block_tables.shape[1] * PAGE)) if split else 0
+    scratch = torch.empty(n, dtype=torch.uint8, device=q.device) if n else None
+    _lib.check(lib.sd_multimap_softmax_attention(
+        _p(q), q.shape[1], _p(k_cache), _p(v_cache), int(k_cache.dtype == torch.float32), _p(row_pos),
+        _p(row_slot), _p(block_tables), block_tables.shape[1], PAGE, q.shape[0], H, G, int(maps), dk, dv, window,
+        int(keep_first), int(chunk), float(scale), float(softcap), _p(sinks), _p(out), None, _p(scratch), n,
+        _stream()), "sd_multimap_softmax_attention")
+    return out
+
+
+def attn_prep(q, k, v, dk, G, dv, row_pos, row_slot, block_tables, k_cache, v_cache, *, q_bias=None, k_bias=None,
+              norm="none", q_norm_w=None, k_norm_w=None, eps=1e-5, rot_dims=0, rot_layout=0, inv_freq=None, mag=1.0):
+    """sd_attn_prep on q f32 [rows, units*dk], k f32 [rows, units*dk] (or None: only q) and v f32
+    [rows, G*dv] (or None: the values are the keys after their bias).  norm: "none", "full" (over
+    the whole projection) or "head" (per unit, one weight [dk]).  Returns the prepared (q, k);
+    keys and values are appended to the caches, whose dtype is the weights'."""
+    _f32(q, "q")
+    parts = [q] + ([k] if k is not None else []) + ([v] if v is not None else [])
+    buf = torch.cat(parts, dim=1).contiguous()
+    nq, nk = q.shape[1], (k.shape[1] if k is not None else 0)
+    typed = next((t for t in (k_cache, q_norm_w, q_bias) if t is not None), None)   # the weights' element type
+    w_f32 = 1 if typed is None else int(typed.dtype == torch.float32)
+    _lib.check(_lib.load().sd_attn_prep(
+        buf.data_ptr(), nq // dk, buf.data_ptr() + 4 * nq if k is not None else None, nk // dk, dk,
+        buf.data_ptr() + 4 * (nq + nk) if v is not None else None, G, dv, int(k is not None and v is None),
+        buf.shape[1], _p(q_bias), _p(k_bias), {"none": 0, "full": 1, "head": 2}[norm], _p(q_norm_w), _p(k_norm_w),
+        w_f32, float(eps), int(rot_dims), int(rot_layout), _p(inv_freq), float(mag), _p(k_cache), _p(v_cache),
+        _p(row_pos), _p(row_slot), _p(block_tables), block_tables.shape[1] if block_tables is not None else 0, PAGE,
+        q.shape[0], _stream()), "sd_attn_prep")
+    return buf[:, :nq].contiguous(), (buf[:, nq:nq + nk].contiguous() if k is not None else None)
+
+
+def diff_combine_rows(a, lam, eps, out_scale, H, dv, bf16_copy=False):
+    """a f32 [rows, H*2*dv] (two maps per head) -> (a1 - lam * a2) / rms * out_scale, f32 [rows, H*dv]."""
+    _f32(a, "a")
+    n = a.shape[0]
+    y = torch.empty(n, H * dv, dtype=torch.float32, device=a.device)
+    yb = torch.empty(n, H * dv, dtype=torch.bfloat16, device=a.device) if bf16_copy else None
+    _lib.check(_lib.load().sd_diff_combine_rows(_p(a), float(lam), float(eps), float(out_scale), _p(y), _p(yb), n, H,
+                                                dv, int(bf16_copy), _stream()), "sd_diff_combine_rows")
+    return (y, yb) if bf16_copy else y
+
+
+def moe_route_rows_biased(x, w_router, router_bias, top, score="softmax", renorm=True, renorm_eps=0.0,
+                          weight_scale=1.0):
+    """moe_route_rows_gated with router_bias f32 [E] added to the logits: (experts, weights, logits)."""
+    _f32(x, "x")
+    _f32(router_bias, "router_bias")
+    n, K = x.shape
+    E = w_router.shape[0]
+    sel_e = torch.empty(n, top, dtype=torch.int32, device=x.device)
+    sel_w = torch.empty(n, top, dtype=torch.float32, device=x.device)
+    logits = torch.empty(n, E, dtype=torch.float32, device=x.device)
+    _lib.check(_lib.load().sd_moe_route_rows_biased(
+        _p(x), K, _p(w_router), _p(router_bias), _wkind(w_router, "w_router"), _p(logits), _p(sel_e), _p(sel_w), n, E,
+        K, top, {"sigmoid": 0, "softmax": 1}[score], int(renorm), float(renorm_eps), float(weight_scale), None, 0,
+        None, _stream()), "sd_moe_route_rows_biased")
+    return sel_e, sel_w, logits
+
+
+def residual_norm_scaled(x, a, w_post, mult, n_a=1, a_bias=None, b=None, w_next=None, eps=1e-5):
+    """sd_residual_norm_scaled, in place on x f32 [rows, W]: x += mult * rms_norm(sum of each row's
+    n_a rows of a + a_bias (+ b)) * w_post; returns rms_norm(x) * w_next if w_next is given."""
+    _f32(x, "x")
+    n, W = x.shape
+    h = torch.empty_like(x) if w_next is not None else None
+    _lib.check(_lib.load().sd_residual_norm_scaled(_p(x), _p(a), int(n_a), _p(a_bias), _p(b), None, 0, _p(w_post),
+                                                   float(mult), None, _p(w_next), _wkind(w_post, "w_post"), float(eps),
+                                                   None, _p(h), None, n, W, _stream()), "sd_residual_norm_scaled")
+    return h
+
+
 def matmul_rows_batched(x, w) -> torch.Tensor:
     """x f32 [M, B, K], w [B, N, K] -> f32 [M, B, N]: product b uses w[b]."""
     _f32(x, "x")
