@@ -102,7 +102,7 @@ def parse():
     ap.add_argument("--tp-draft", choices=["replicated", "sharded"], default="replicated",
                     help="the draft whole on every rank (no exchange in its passes), or sharded "
                          "like the target with a vocabulary-parallel head")
-    ap.add_argument("--family", choices=["spec", "puguzen", "naburax", "fepopel"], default="spec",
+    ap.add_argument("--family", choices=["spec", "puguzen", "naburax", "fepopel", "zopupel"], default="spec",
                     help="spec: the headline speculative-decoding workload (default).  puguzen: prefill and "
                          "decode throughput of the Puguzen decoder family (recurrent and windowed layers) at "
                          "layer sizes of real models, beside a Llama-style decoder of equal size, with the "
@@ -111,8 +111,12 @@ def parse():
                          "experts), beside the Puguzen family at equal size.  fepopel: the same for the "
                          "Fepopel family (latent attention with a sink over every earlier token, chunked "
                          "softmax attention, experts of two matrices beside a shared one, a repeated span of "
-                         "layers), beside the Naburax family at equal size")
-    ap.add_argument("--seq-sizes", default="w1024,w2048,w4096", help="--family puguzen / naburax / fepopel: sizes to run")
+                         "layers), beside the Naburax family at equal size.  zopupel: the same for the "
+                         "Zopupel family (differential attention with shared keys and values, attention whose "
+                         "values are its keys, gated experts with a router bias beside a shared one), beside "
+                         "the Fepopel family at equal size")
+    ap.add_argument("--seq-sizes", default="w1024,w2048,w4096",
+                    help="--family puguzen / naburax / fepopel / zopupel: sizes to run")
     return ap.parse_args()
 
 
@@ -1086,8 +1090,149 @@ def main_fep_family(args):
                       "data": "synthetic", "n_gpus": 1, "steps": steps, "warmup": warm, "sizes": results}))
 
 
+# ---------------------------------------------------------------------------------------------
+# --family zopupel
+ZOP_SIZES = {
+    "w1024": dict(width=1024, heads=8, kv_heads=2, experts=8, top=2, eff=1024, shared=1024),
+    "w2048": dict(width=2048, heads=16, kv_heads=4, experts=16, top=2, eff=2048, shared=2048),
+    "w4096": dict(width=4096, heads=32, kv_heads=8, experts=16, top=2, eff=4096, shared=4096),
+}
+ZOP_BLEND = {"factor": 8.0, "original": 4096, "fast": 32.0, "slow": 1.0}
+
+
+def _zop_config(sz):
+    """Six layers as the Fepopel bench model has six layer runs: attention whose values are its
+    keys (heads of SEQ_HEAD channels) and differential attention (two maps of SEQ_HEAD / 2 channels
+    per head over values of SEQ_HEAD channels), the second differential layer reading the first
+    one's keys and values; every layer with routed gated experts beside a shared one."""
+    from vllm_omni_draft_amd.config import ExpertsSpec, MixerSpec, SeqLayerSpec, SeqModelConfig
+    H, G, D = sz["heads"], sz["kv_heads"], SEQ_HEAD
+    kv = MixerSpec("softmax_attention", H, D, D, kv_heads=G, scale=D ** -0.5, window=0, rot_dims=D // 2, rot_base=1e6,
+                   rot_layout="half", rot_scaling=dict(ZOP_BLEND), qk_full_norm=True, proj_bias=True,
+                   value_is_key=True, unit_sink=True)
+    df = dict(kind="softmax_attention", heads=H, dim=D // 2, vdim=D, kv_heads=G, scale=(D // 2) ** -0.5, window=0,
+              rot_dims=D // 2, rot_base=1e6, rot_layout="half", rot_scaling={"factor": 4.0}, maps=2, diff=0.3)
+    ex = ExpertsSpec(sz["experts"], sz["top"], sz["eff"], score="softmax", renorm=True, scale_input=False, act="silu",
+                     shared_ff=sz["shared"], shared_gate=False, router_bias=True)
+    mixers = [kv, MixerSpec(**df), kv, kv, MixerSpec(kv_from=1, **df), kv]
+    cfg = SeqModelConfig("zopupel", sz["width"], SEQ_VOCAB, [SeqLayerSpec(m, 0, ex, ff_act="silu") for m in mixers],
+                         name="zopupel-bench", block="sandwich", tied_head=False, residual_mult=0.3)
+    cfg.validate()
+    return cfg
+
+
+def zop_kernel_rooflines(cfg, device, ctx, rows):
+    """The family's own kernels alone at `rows` token rows of one sequence that ends at position
+    ctx, as fep_kernel_rooflines reports them; `like` names the Fepopel kernel each is set beside."""
+    from vllm_omni_draft_amd import ops
+    kv = next(l.mixer for l in cfg.layers if l.mixer.value_is_key)
+    df = next(l.mixer for l in cfg.layers if l.mixer.maps == 2)
+    ex, W = cfg.layers[0].experts, cfg.width
+    g = torch.Generator(device="cpu").manual_seed(0)
+    rn = lambda *s: torch.randn(*s, generator=g).to(device)
+    bf = lambda *s: torch.randn(*s, generator=g).to(torch.bfloat16).to(device)
+    pages = -(-ctx // ops.PAGE)
+    tables = torch.arange(pages, dtype=torch.int32, device=device).view(1, -1)
+    pos_l = list(range(ctx - rows, ctx))
+    pos = torch.tensor(pos_l, dtype=torch.int32, device=device)
+    slot = torch.zeros(rows, dtype=torch.int32, device=device)
+    keys = sum(p + 1 for p in pos_l)
+    out = []
+    # differential attention: two maps of dk channels per head over every earlier token, one value row per kv head
+    H, G, dk, dv = df.heads, df.kv_heads, df.dim, df.vdim
+    kc, vc = bf(pages, G * 2, ops.PAGE, dk), bf(pages, G, ops.PAGE, dv)
+    q = rn(rows, H * 2 * dk)
+    us = _events(lambda: ops.multimap_softmax_attention(q, kc, vc, pos, slot, tables, H, G, 2, dk, dv, df.scale), 5)
+    out.append(("multimap_softmax_attention (two maps, all keys)", "masked_softmax_attention (grouped heads, chunks, cap)",
+                us, G * 2 * (2 * dk + dv) * ctx + 4 * rows * H * 2 * (dk + dv), 2.0 * keys * H * 2 * (dk + dv),
+                F32_VALU_PEAK_TFLOPS))
+    a2 = rn(rows, H * 2 * dv)
+    us = _events(lambda: ops.diff_combine_rows(a2, 0.4, 1e-6, 0.7, H, dv, bf16_copy=True), 5)
+    out.append(("diff_combine_rows", "", us, rows * H * dv * (8 + 4 + 2), 0.0, F32_VALU_PEAK_TFLOPS))
+    # attention whose values are its keys as projected, one more term in the denominator
+    H, G, D = kv.heads, kv.kv_heads, kv.dim
+    kc2, vc2 = bf(pages, G, ops.PAGE, D), bf(pages, G, ops.PAGE, D)
+    q2, sinks = rn(rows, H * D), torch.zeros(H, device=device)
+    us = _events(lambda: ops.multimap_softmax_attention(q2, kc2, vc2, pos, slot, tables, H, G, 1, D, D, kv.scale,
+                                                        sinks=sinks), 5)
+    out.append(("multimap_softmax_attention (one map, all keys, unit term)",
+                "masked_softmax_attention (grouped heads, chunks, cap)", us, G * 2 * D * 2 * ctx + 8 * rows * H * D,
+                2.0 * keys * H * 2 * D, F32_VALU_PEAK_TFLOPS))
+    # the preparation: biases, norms over the whole projection, rotary turn, append of keys and of the keys as values
+    from vllm_omni_draft_amd.config import rotary_frequencies
+    f, mag = rotary_frequencies(kv.rot_dims, kv.rot_base, kv.rot_scaling)
+    f = f.to(device)
+    qp, kp = rn(rows, H * D), rn(rows, G * D)
+    qb, kb, qw, kw = bf(H * D), bf(G * D), bf(H * D), bf(G * D)
+    us = _events(lambda: ops.attn_prep(qp, kp, None, D, G, D, pos, slot, tables, kc2, vc2, q_bias=qb, k_bias=kb,
+                                       norm="full", q_norm_w=qw, k_norm_w=kw, eps=1e-6, rot_dims=kv.rot_dims,
+                                       inv_freq=f, mag=mag), 5)
+    # (the wrapper stacks q and k into one buffer and splits them again: its copies are inside the time)
+    out.append(("attn_prep (wrapper copies included)", "qk_head_norm_append", us,
+                8 * rows * (H + G) * D + 2 * rows * 2 * G * D, 0.0, F32_VALU_PEAK_TFLOPS))
+    # routed gated experts (grouping, gate / up, down), weights on the outputs
+    E, top, F = ex.experts, ex.top, ex.ff
+    x = rn(rows, W)
+    gu = (torch.randn(E, 2 * F, W, generator=g) * W ** -0.5).to(torch.bfloat16).to(device)
+    dn = (torch.randn(E, W, F, generator=g) * F ** -0.5).to(torch.bfloat16).to(device)
+    sel_e = torch.stack([torch.randperm(E, generator=g)[:top] for _ in range(rows)]).to(torch.int32).to(device)
+    sel_w = torch.rand(rows, top, generator=g).to(device)
+    us = _events(lambda: ops.moe_experts(x, sel_e, sel_w, gu, dn, scale_input=False, act="silu"), 5)
+    used = min(E, rows * top)
+    out.append(("moe_experts (gated)", "moe_experts (two matrices)", us,
+                2 * used * 3 * F * W + 4 * rows * W * (1 + top) + 2 * rows * top * F * 2,
+                2.0 * rows * top * 3 * F * W, BF16_MFMA_PEAK_TFLOPS))
+    wr, rb = (torch.randn(E, W, generator=g) * W ** -0.5).to(torch.bfloat16).to(device), rn(E)
+    us = _events(lambda: ops.moe_route_rows_biased(x, wr, rb, top), 5)
+    out.append(("moe_route_rows_biased", "moe_route_rows_gated", us, 4 * rows * W + 2 * E * W, 2.0 * rows * E * W,
+                F32_VALU_PEAK_TFLOPS))
+    # residual update with the output matrix's bias, the factor, and the norms around it
+    a, b = rn(rows * top, W), rn(rows, W)
+    wp, wn, ab = bf(W), bf(W), bf(W)
+    xr = rn(rows, W)
+    us = _events(lambda: ops.residual_norm_scaled(xr, a, wp, 0.3, n_a=top, a_bias=ab, b=b, w_next=wn, eps=1e-6), 5)
+    out.append(("residual_norm_scaled", "residual_norm", us, 4 * rows * W * (top + 1 + 2 + 1) + 2 * rows * W, 0.0,
+                F32_VALU_PEAK_TFLOPS))
+    res = []
+    for name, like, us, nbytes, flops, peak in out:
+        floor_us = max(nbytes / (HBM_PEAK_GBS * 1e3), flops / (peak * 1e6))
+        res.append({"kernel": name, "like": like, "rows": rows, "ctx": ctx, "avg_us": round(us, 2),
+                    "min_bytes": int(nbytes), "flops": int(flops), "achieved_gbs": round(nbytes / us * 1e-3, 1),
+                    "achieved_tflops": round(flops / us * 1e-6, 2), "roofline_us": round(floor_us, 2),
+                    "times_roofline": round(us / floor_us, 1)})
+    return res
+
+
+def main_zop_family(args):
+    """Prefill and decode throughput of the Zopupel family beside the Fepopel family at equal
+    width, heads and expert width (both bf16, seeded random weights), one JSON line."""
+    if not torch.cuda.is_available():
+        raise SystemExit("bench.py needs a GPU (there is no CPU path)")
+    device = torch.device("cuda", 0)
+    P, B, steps, warm = args.prompt_len, 4, args.steps, args.warmup
+    results = []
+    for name in args.seq_sizes.split(","):
+        sz = ZOP_SIZES[name]
+        cfg = _zop_config(sz)
+        mine = _run_seq_engine(cfg, device, P, B, steps, warm)
+        mine["layer_runs"] = cfg.n_runs
+        kern = zop_kernel_rooflines(cfg, device, P, 1) + zop_kernel_rooflines(cfg, device, P, min(P, 1024))
+        fcfg = _fep_config(FEP_SIZES[name])
+        other = _run_seq_engine(fcfg, device, P, B, steps, warm)
+        other["layer_runs"] = fcfg.n_runs
+        like = fep_kernel_rooflines(fcfg, device, P, 1) + fep_kernel_rooflines(fcfg, device, P, min(P, 1024))
+        results.append({"size": name, **sz, "layers": ["diff" if l.mixer.maps == 2 else "keyval" for l in cfg.layers],
+                        "head_dim": SEQ_HEAD, "prompt_len": P, "decode_batch": B, "zopupel": mine,
+                        "fepopel_equal_size": other, "kernels": kern, "fepopel_kernels": like})
+    print(json.dumps({"metric": "zopupel_family_throughput", "unit": "tokens/s", "dtype": "bf16",
+                      "data": "synthetic", "n_gpus": 1, "steps": steps, "warmup": warm, "sizes": results}))
+
+
 def main():
     args = parse()
+    if args.family == "zopupel":
+        main_zop_family(args)
+        return
     if args.family == "fepopel":
         main_fep_family(args)
         return

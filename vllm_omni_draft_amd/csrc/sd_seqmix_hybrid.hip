@@ -603,8 +603,15 @@ template <typename T>
 __device__ __forceinline__ void prep_units(float* __restrict__ x, int n_units, int dk, const T* __restrict__ bias,
                                            int norm_kind, const T* __restrict__ w, float eps, int dims, int layout,
                                            const double* __restrict__ inv_freq, float mag, int pos, float* red,
-                                           T* __restrict__ raw_dst_base, int raw_dv, size_t raw_head_stride) {
+                                           T* __restrict__ raw_dst_base, int raw_dv, size_t raw_head_stride,
+                                           float* __restrict__ cs) {
   const int n = n_units * dk;
+  // the row's cosines and sines once, for every unit (the angle is formed in f64)
+  for (int i = threadIdx.x; i < dims / 2; i += blockDim.x) {
+    const double a = (double)pos * inv_freq[i];
+    cs[i] = (float)cos(a) * mag;
+    cs[dims / 2 + i] = (float)sin(a) * mag;
+  }
   float ss = 0.f;
   for (int c = threadIdx.x; c < n; c += blockDim.x) {
     float v = x[c];
@@ -622,22 +629,25 @@ __device__ __forceinline__ void prep_units(float* __restrict__ x, int n_units, i
   }
   __syncthreads();
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, nw = blockDim.x >> 6;
-  for (int u = wave; u < n_units; u += nw) {     // a wave per unit
-    float* xu = x + (size_t)u * dk;
-    if (norm_kind == 2) {
+  if (norm_kind == 2) {
+    for (int u = wave; u < n_units; u += nw) {   // a wave per unit
+      float* xu = x + (size_t)u * dk;
       float s2 = 0.f;
       for (int c = lane; c < dk; c += 64) s2 = fmaf(xu[c], xu[c], s2);
       s2 = wave_sum(s2);
       const float rstd = 1.f / sqrtf(s2 / (float)dk + eps);
       for (int c = lane; c < dk; c += 64) xu[c] = xu[c] * rstd * ld_f(w + c);
     }
+    __syncthreads();
+  }
+  for (int u = wave; u < n_units; u += nw) {     // a wave per unit
+    float* xu = x + (size_t)u * dk;
     for (int i = lane; i < dims / 2; i += 64) {
-      const double a = (double)pos * inv_freq[i];
-      const float cs = (float)cos(a) * mag, sn = (float)sin(a) * mag;
+      const float c = cs[i], sn = cs[dims / 2 + i];
       const int iu = layout ? 2 * i : i, iv = layout ? 2 * i + 1 : i + dims / 2;
       const float p = xu[iu], q = xu[iv];
-      xu[iu] = p * cs - q * sn;
-      xu[iv] = q * cs + p * sn;
+      xu[iu] = p * c - q * sn;
+      xu[iv] = q * c + p * sn;
     }
   }
 }
@@ -649,12 +659,13 @@ __global__ __launch_bounds__(256) void attn_prep_kernel(
     const double* __restrict__ inv_freq, float mag, const int32_t* __restrict__ row_pos,
     const int32_t* __restrict__ row_slot, const int32_t* __restrict__ block_tables, int max_blocks, int page,
     T* __restrict__ k_cache, T* __restrict__ v_cache) {
+  extern __shared__ float cs[];   // [dims]: cosines, then sines
   __shared__ float red[4];
   const int r = blockIdx.x;
   const int pos = row_pos[r];
   if (blockIdx.y == 0) {
     prep_units<T>(q + (size_t)r * ld, nq, dk, q_bias, norm_kind, q_w, eps, dims, layout, inv_freq, mag, pos, red,
-                  nullptr, 1, 0);
+                  nullptr, 1, 0, cs);
     return;
   }
   const int pg = block_tables[(size_t)row_slot[r] * max_blocks + pos / page];
@@ -662,7 +673,7 @@ __global__ __launch_bounds__(256) void attn_prep_kernel(
   // (cache rows of one token: head g at ((pg * heads + g) * page + pos % page) * channels)
   T* v_dst = v_cache + ((size_t)pg * G * page + pos % page) * dv;
   prep_units<T>(kr, nk, dk, k_bias, norm_kind, k_w, eps, dims, layout, inv_freq, mag, pos, red,
-                v_from_k ? v_dst : nullptr, dv, (size_t)page * dv);
+                v_from_k ? v_dst : nullptr, dv, (size_t)page * dv, cs);
   __syncthreads();
   for (int c = threadIdx.x; c < nk * dk; c += blockDim.x)
     st_f(k_cache + (((size_t)pg * nk + c / dk) * page + pos % page) * dk + c % dk, kr[c]);
@@ -1840,13 +1851,13 @@ extern "C" int sd_attn_prep(float* q, int n_q_units, float* k, int n_k_units, in
   hipStream_t st = (hipStream_t)stream;
   const dim3 grid(n_rows, k ? 2 : 1);
   if (w_f32)
-    attn_prep_kernel<float><<<grid, 256, 0, st>>>(q, n_q_units, k, n_k_units, dk, v, G, dv, value_from_key, ld,
+    attn_prep_kernel<float><<<grid, 256, sizeof(float) * (rot_dims > 0 ? rot_dims : 1), st>>>(q, n_q_units, k, n_k_units, dk, v, G, dv, value_from_key, ld,
                                                   (const float*)q_bias, (const float*)k_bias, norm_kind,
                                                   (const float*)q_norm_w, (const float*)k_norm_w, eps, rot_dims,
                                                   rot_layout, inv_freq, mag, row_pos, row_slot, block_tables,
                                                   max_blocks, page, (float*)k_cache, (float*)v_cache);
   else
-    attn_prep_kernel<bf16_t><<<grid, 256, 0, st>>>(q, n_q_units, k, n_k_units, dk, v, G, dv, value_from_key, ld,
+    attn_prep_kernel<bf16_t><<<grid, 256, sizeof(float) * (rot_dims > 0 ? rot_dims : 1), st>>>(q, n_q_units, k, n_k_units, dk, v, G, dv, value_from_key, ld,
                                                    (const bf16_t*)q_bias, (const bf16_t*)k_bias, norm_kind,
                                                    (const bf16_t*)q_norm_w, (const bf16_t*)k_norm_w, eps, rot_dims,
                                                    rot_layout, inv_freq, mag, row_pos, row_slot, block_tables,
