@@ -35,7 +35,13 @@ $(LIB): $(OBJS)
 # run in a fresh checkout that should not wait for every kernel family to compile.  The package
 # loads it only where the whole library has not been built.
 SEQ_LIB  := vllm_omni_draft_amd/libsd_seq.so
-SEQ_OBJS := $(CSRC)/sd_base.o $(CSRC)/sd_seqmix.o $(CSRC)/sd_seqmix_hybrid.o $(CSRC)/sd_sampling.o $(CSRC)/sd_linear.o $(CSRC)/sd_linear_wide.o
+# (these models call the many-row linear family with bf16 weights and its f32 epilogue only: that file is
+# compiled for them without its other instantiations, which take most of the whole library's build time)
+# (... and in two parts side by side, the kernels of few and of many token tiles)
+SEQ_OBJS := $(CSRC)/sd_base.o $(CSRC)/sd_seqmix.o $(CSRC)/sd_seqmix_hybrid.o $(CSRC)/sd_sampling.o $(CSRC)/sd_linear.o \
+	$(CSRC)/sd_linear_wide_seq1.o $(CSRC)/sd_linear_wide_seq2.o
+$(CSRC)/sd_linear_wide_seq%.o: $(CSRC)/sd_linear_wide.hip $(CSRC)/sd_common.h include/sd_amd.h
+	$(HIPCC) $(FLAGS) -DSD_WIDE_F32_ONLY -DSD_WIDE_PART=$* -c $< -o $@
 $(SEQ_LIB): $(SEQ_OBJS)
 	$(HIPCC) --offload-arch=$(ARCH) -shared -fPIC -o $@ $(SEQ_OBJS)
 seq: $(SEQ_LIB)

@@ -1008,9 +1008,11 @@ int launch_gemm_a8(const WideArgs& a, int S, hipStream_t st) {
   }
 }
 
+// SD_WIDE_F32_ONLY: the build for the library of layer-list models alone, which call this family
+// with bf16 weights and the f32 epilogue only; everything else answers SD_ERR_UNSUPPORTED there.
 template <int MT, int EPI, int TPW>
 int launch_gemm_t(const WideArgs& a, int S, hipStream_t st) {
-#ifdef SD_WIDE_EXP  // experiments: a quick build of the few instantiations under study
+#if defined(SD_WIDE_EXP) || defined(SD_WIDE_F32_ONLY)  // a quick build of the few instantiations needed
   return launch_gemm_w<MT, EPI, TPW, false>(a, S, st);
 #else
   return a.epi.w_scale ? launch_gemm_w<MT, EPI, TPW, true>(a, S, st)
@@ -1040,7 +1042,7 @@ int launch_gemm4_w(const WideArgs& a, int S, hipStream_t st) {
 
 template <int MT, int EPI, int TPW, int WAVES>
 int launch_gemm4(const WideArgs& a, int S, hipStream_t st) {
-#ifdef SD_WIDE_EXP
+#if defined(SD_WIDE_EXP) || defined(SD_WIDE_F32_ONLY)
   return launch_gemm4_w<MT, EPI, TPW, false, WAVES>(a, S, st);
 #else
   return a.epi.w_scale ? launch_gemm4_w<MT, EPI, TPW, true, WAVES>(a, S, st)
@@ -1056,7 +1058,7 @@ int g_wide_four_waves = -1;  // experiments: -1 the library's choice, 0 never th
 template <int MT, int EPI>
 int launch_gemm(const WideArgs& a, int S, hipStream_t st) {
   const bool pair = a.group_tiles != kWideWaves;  // 16-tile groups
-#ifndef SD_WIDE_EXP
+#if !defined(SD_WIDE_EXP) && !defined(SD_WIDE_F32_ONLY)
   if (a.x_inv) return pair ? launch_gemm_a8<MT, EPI, 2>(a, S, st) : launch_gemm_a8<MT, EPI, 1>(a, S, st);
 #endif
   // The four-wave kernel where it was measured faster (same bits either way): many rows,
@@ -1101,13 +1103,15 @@ int launch_epi(const WideEpiArgs& e, hipStream_t st) {
 
 int epilogue_by_kind(const WideEpiArgs& e, int epi, hipStream_t st) {
   switch (epi) {
+    case SD_EPI_F32: return launch_epi<SD_EPI_F32>(e, st);
+#ifndef SD_WIDE_F32_ONLY
     case SD_EPI_STORE: return launch_epi<SD_EPI_STORE>(e, st);
     case SD_EPI_RESIDUAL: return launch_epi<SD_EPI_RESIDUAL>(e, st);
     case SD_EPI_SILU_MUL: return launch_epi<SD_EPI_SILU_MUL>(e, st);
     case SD_EPI_RELU: return launch_epi<SD_EPI_RELU>(e, st);
-    case SD_EPI_F32: return launch_epi<SD_EPI_F32>(e, st);
     case SD_EPI_GELU_TANH: return launch_epi<SD_EPI_GELU_TANH>(e, st);
     case EPI_QKV_ROPE: return launch_epi<EPI_QKV_ROPE>(e, st);
+#endif
   }
   sd_set_error("sd_linear_wide: unknown epilogue %d", epi);
   return SD_ERR_INVALID;
@@ -1116,6 +1120,11 @@ int epilogue_by_kind(const WideEpiArgs& e, int epi, hipStream_t st) {
 template <int MT, bool DIRECT>
 int gemm_by_kind(const WideArgs& a, int epi, int S, hipStream_t st) {
   if (!DIRECT) return launch_gemm<MT, EPI_PARTIAL>(a, S, st);
+#ifdef SD_WIDE_F32_ONLY
+  if (epi == SD_EPI_F32) return launch_gemm<MT, SD_EPI_F32>(a, S, st);
+  sd_set_error("sd_linear_wide: epilogue %d is not in the library of layer-list models alone", epi);
+  return SD_ERR_UNSUPPORTED;
+#endif
   switch (epi) {
     case SD_EPI_STORE: return launch_gemm<MT, SD_EPI_STORE>(a, S, st);
     case SD_EPI_RESIDUAL: return launch_gemm<MT, SD_EPI_RESIDUAL>(a, S, st);
@@ -1131,9 +1140,26 @@ int gemm_by_kind(const WideArgs& a, int epi, int S, hipStream_t st) {
   return SD_ERR_INVALID;
 }
 
+}  // namespace
+#ifdef SD_WIDE_F32_ONLY
+// The build for layer-list models compiles this file twice, side by side: SD_WIDE_PART 1 holds the
+// entry points and the kernels of up to 8 token tiles, SD_WIDE_PART 2 only the kernels of 12 and 16
+// token tiles behind this function (args: the WideArgs of the call).
+extern "C" int sd_wide_rows_upper_(const void* args, int mt, int epi, int S, void* stream, int direct);
+#endif
+namespace {
+
 template <bool DIRECT>
 int gemm_by_rows(const WideArgs& a, int mt, int epi, int S, hipStream_t st) {
-#ifdef SD_WIDE_EXP
+#if defined(SD_WIDE_F32_ONLY) && SD_WIDE_PART == 1
+  if (mt > 8) return sd_wide_rows_upper_(&a, mt, epi, S, st, DIRECT ? 1 : 0);
+  if (mt <= 2) return gemm_by_kind<2, DIRECT>(a, epi, S, st);
+  if (mt <= 4) return gemm_by_kind<4, DIRECT>(a, epi, S, st);
+  return gemm_by_kind<8, DIRECT>(a, epi, S, st);
+#elif defined(SD_WIDE_F32_ONLY)
+  if (mt <= 12) return gemm_by_kind<12, DIRECT>(a, epi, S, st);
+  return gemm_by_kind<16, DIRECT>(a, epi, S, st);
+#elif defined(SD_WIDE_EXP)
 #ifndef SD_WIDE_EXP_MT
 #define SD_WIDE_EXP_MT 12
 #endif
@@ -1147,10 +1173,25 @@ int gemm_by_rows(const WideArgs& a, int mt, int epi, int S, hipStream_t st) {
 #endif
 }
 
+#if defined(SD_WIDE_F32_ONLY) && SD_WIDE_PART == 2
+}  // namespace
+extern "C" int sd_wide_rows_upper_(const void* args, int mt, int epi, int S, void* stream, int direct) {
+  const WideArgs& a = *static_cast<const WideArgs*>(args);
+  return direct ? gemm_by_rows<true>(a, mt, epi, S, (hipStream_t)stream)
+                : gemm_by_rows<false>(a, mt, epi, S, (hipStream_t)stream);
+}
+namespace {
+#endif
+
+#if !defined(SD_WIDE_F32_ONLY) || SD_WIDE_PART == 1
 int wide_common(const void* W, const void* x, int64_t ldx, int M, int K, int n_tiles, int epi,
                 WideEpiArgs& e, void* workspace, size_t ws_bytes, hipStream_t st,
                 const float* x_scales = nullptr) {
   SD_REQUIRE(W && x && e.out && workspace, SD_ERR_INVALID, "sd_linear_wide: null pointer");
+#ifdef SD_WIDE_F32_ONLY
+  SD_REQUIRE(!e.w_scale && !x_scales && epi == SD_EPI_F32, SD_ERR_UNSUPPORTED,
+             "sd_linear_wide: fp8 operands and epilogue %d are not in the library of layer-list models alone", epi);
+#endif
   SD_REQUIRE(M >= 0 && M <= 256, SD_ERR_UNSUPPORTED, "sd_linear_wide: M=%d outside 0..256", M);
   SD_REQUIRE(K >= 32 && K % 32 == 0 && n_tiles >= 1, SD_ERR_INVALID,
              "sd_linear_wide: K must be a positive multiple of 32 (K=%d)", K);
@@ -1185,9 +1226,11 @@ int wide_common(const void* W, const void* x, int64_t ldx, int M, int K, int n_t
   if (rc != SD_OK) return rc;
   return epilogue_by_kind(e, epi, st);
 }
+#endif
 
 }  // namespace
 
+#if !defined(SD_WIDE_F32_ONLY) || SD_WIDE_PART == 1
 extern "C" size_t sd_linear_wide_workspace_bytes(int M, int N, int K, int epilogue) {
   if (M < 1 || N < 1 || K < 32 || K % 32) return 0;
   return wide_ws_bytes(M, tiles_of(N, epilogue), K);
@@ -1308,3 +1351,4 @@ extern "C" int sd_debug_read_wide_stamps(unsigned long long* host) {
   return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(sd_wide_stamps), sizeof(sd_wide_stamps));
 }
 #endif
+#endif  // the entry points: not in the second part of the build for layer-list models
