@@ -565,3 +565,38 @@ def test_greedy_generation_through_worker_and_scheduler():
                 assert (top[0] - top[1]) / logits.std() < 1e-4
                 break
             toks.append(tok)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_replay_command_line(tmp_path, dtype):
+    """bin/trace_run on a checkpoint folder: the class chosen by config.json, steps read from
+    standard input (portions beside single tokens, requests ended and their pages used again by a
+    pool that holds two requests at most), logits written per step."""
+    import json
+    import os
+    import subprocess
+    import sys
+    import numpy as np
+    from safetensors.torch import save_file
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    cfg = SHAPES["two_kinds"]
+    st = {k: v.to(torch.bfloat16).float() for k, v in Z.random_tensors(cfg, 6).items()}
+    model, out = tmp_path / "model", tmp_path / "out"
+    model.mkdir()
+    (model / "config.json").write_text(json.dumps(cfg))
+    save_file({k: v.to(torch.bfloat16).contiguous() for k, v in st.items()}, str(model / "model.safetensors"))
+    pa, pb, pc = prompt(cfg, 70, 1), prompt(cfg, 50, 2), prompt(cfg, 64, 3)
+    steps = [{"step": 0, "entries": [{"id": "a", "tokens": pa[:33], "want": [0, 32]}], "end": []},
+             {"step": 1, "entries": [{"id": "a", "tokens": pa[33:35], "want": [1]}, {"id": "b", "tokens": pb[:49], "want": []}], "end": []},
+             {"step": 2, "entries": [{"id": "b", "tokens": pb[49:], "want": [0]}], "end": ["b"]},
+             {"step": 3, "entries": [{"id": "a", "tokens": pa[35:], "want": [34]}, {"id": "c", "tokens": pc, "want": [63]}], "end": ["a", "c"]}]
+    run = subprocess.run([sys.executable, os.path.join(root, "bin", "trace_run"), "--model", str(model), "--dtype", dtype,
+                          "--out", str(out), "--max-tokens", "192"], input="".join(json.dumps(s) + "\n" for s in steps),
+                         capture_output=True, text=True, timeout=300)
+    assert run.returncode == 0, run.stderr[-2000:]
+    assert [l for l in run.stdout.splitlines() if l.startswith("done")] == ["done 0", "done 1", "done 2", "done 3"]
+    wa, wb, wc = (Z.forward(cfg, st, p) for p in (pa, pb, pc))
+    want = {0: wa[[0, 32]], 1: wa[[34]], 2: wb[[49]], 3: torch.stack([wa[69], wc[63]])}
+    for n, w in want.items():
+        got = torch.from_numpy(np.fromfile(str(out / f"{n}.f32"), dtype="<f4").reshape(w.shape[0], cfg["vocab"]).copy())
+        assert rel(got, w) < (3e-6 if dtype == "float32" else 5e-2), n
